@@ -31,13 +31,19 @@ class LayerSpec:
     prefix: str                 # e.g. "model.layers.3."
     block: str                  # arrangement of the parts, e.g. "pre_norm"
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: PartSpec | None
     mixer_norm: PartSpec        # the norm in front of the mixer
     feed_forward_norm: PartSpec  # the norm in front of the feed-forward
     mixer_norm_place: str = "input_layernorm."
     mixer_place: str = "self_attn."
     feed_forward_norm_place: str = "post_attention_layernorm."
     feed_forward_place: str = "mlp."
+    # for arrangements that also norm a sublayer's result before it joins the residual ("sandwich_norm"):
+    # those norms and their places; such a layer may also have no feed-forward at all (feed_forward None)
+    mixer_post_norm: PartSpec | None = None
+    feed_forward_post_norm: PartSpec | None = None
+    mixer_post_norm_place: str = "post_mixer_layernorm."
+    feed_forward_post_norm_place: str = "post_feedforward_layernorm."
 
 
 @dataclass(frozen=True)
@@ -58,7 +64,7 @@ class ModelSpec:
     architecture: str
     hidden_size: int
     vocab_size: int
-    max_positions: int
+    max_positions: int | None      # None: the architecture sets no bound (the cache pool's size is the only one)
     embedding: PartSpec
     layers: tuple[LayerSpec, ...]
     runs: tuple[Run, ...]
@@ -94,5 +100,5 @@ class TensorSpec:
     """A tensor a part expects in the checkpoint: its full name, shape and kind of values."""
     name: str
     shape: tuple[int, ...]
-    init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "zeros"
+    init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "offset" (a norm's weight stored around 0), "zeros"
     optional: bool = False       # absent is no error, present it is checked and not read (a tied head's matrix that some files still carry)

@@ -17,10 +17,15 @@
 
 namespace tlie {
 
-// q: [tokens][nq][d]; cache: [pages][2][nkv][page_size * d], keys [row][dim], values [dim][row];
-// out: [tokens][nq][d].
+// q: [tokens][nq][d]; a page of the cache holds nkv planes of keys, [row][d], and after them nkv planes
+// of values, transposed, [dv][row] (with dv = d that is [pages][2][nkv][page_size * d]);
+// out: [tokens][nq][dv].
 // token_seq[t]: row of the block table; positions[t]: absolute position of the token.
 // window <= 0: all keys 0..pos; otherwise keys pos-window+1..pos.
+// chunk > 0: only keys of the query's own chunk of positions, pos - pos % chunk .. pos (chunks are
+// counted from position 0 of the sequence).
+// sink (or null): one number per query head that joins the softmax's denominator as exp(sink): it has
+// no key and no value and is not scaled.
 // A workgroup of 256 threads serves one (token, head).  Its threads form 256 / CHUNK groups of
 // CHUNK threads (CHUNK >= d); chunk c of the context (keys c * CHUNK ..) belongs to group
 // c % groups, and every group keeps a running maximum, sum and output of its own over its chunks,
@@ -33,7 +38,8 @@ template <typename T, int CHUNK>
 __global__ void __launch_bounds__(256)
 attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
                          int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
-                         T* __restrict__ out, int nq, int nkv, int d, int page_size, int window, float scale,
+                         T* __restrict__ out, int nq, int nkv, int d, int dv, int page_size, int window, int chunk,
+                         const float* __restrict__ sink, float scale,
                          const int* __restrict__ seq_start, int min_tokens) {
   constexpr int kGroups = 256 / CHUNK, kWavesPerGroup = CHUNK / 64;
   if (seq_start != nullptr) {                      // (the same for the whole workgroup)
@@ -45,17 +51,18 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
   float* prob = q_row + d;                         // 256: a group's probabilities of its current chunk
   float* wave_part = prob + 256;                   // 4: one value per wave, for the reductions within a group
   float* group_stat = wave_part + 4;               // kGroups x 2: maximum, sum
-  float* group_out = group_stat + 2 * kGroups;     // kGroups x d
+  float* group_out = group_stat + 2 * kGroups;     // kGroups x dv
   const int t = blockIdx.x, h = blockIdx.y;
   const int group = threadIdx.x / CHUNK, place = threadIdx.x % CHUNK;       // place: key of the chunk, then dim of the output
   const int wave = threadIdx.x / 64, first_wave = group * kWavesPerGroup;
   const int kv_head = h / (nq / nkv);
   const int pos = positions[t];
   const int* pages = block_table + static_cast<size_t>(token_seq[t]) * max_blocks;
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const size_t page_stride = static_cast<size_t>(2) * nkv * page_size * d;
+  int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  if (chunk > 0) lo = max(lo, pos - pos % chunk);
+  const size_t page_stride = static_cast<size_t>(nkv) * page_size * (d + dv);
   const size_t head_offset = static_cast<size_t>(kv_head) * page_size * d;
-  const size_t v_offset = static_cast<size_t>(nkv) * page_size * d;
+  const size_t v_offset = static_cast<size_t>(nkv) * page_size * d + static_cast<size_t>(kv_head) * page_size * dv;
 
   for (int i = threadIdx.x; i < d; i += 256) q_row[i] = to_float(q[(static_cast<size_t>(t) * nq + h) * d + i]);
   __syncthreads();
@@ -111,7 +118,7 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
     const float alpha = new_max == -INFINITY ? 1.f : expf(running_max - new_max);   // 0 when this chunk is the group's first with keys
     running_sum = running_sum * alpha + chunk_sum;
     running_max = new_max;
-    if (place < d) {
+    if (place < dv) {
       acc *= alpha;
       const int first = max(0, lo - start), last = min(CHUNK, pos - start + 1);
       int jj = first;
@@ -120,7 +127,7 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
         // 64 and pages hold a multiple of four rows; the additions stay in the order of the keys)
         for (; jj < last && (jj & 3) != 0; ++jj) {
           const int key_pos = start + jj;
-          const T* value = cache + static_cast<size_t>(pages[key_pos / page_size]) * page_stride + v_offset + head_offset +
+          const T* value = cache + static_cast<size_t>(pages[key_pos / page_size]) * page_stride + v_offset +
                            static_cast<size_t>(place) * page_size + key_pos % page_size;
           acc += prob[group * CHUNK + jj] * to_float(*value);
         }
@@ -128,7 +135,7 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
         for (; jj + 4 <= last; jj += 4) {
           const int key_pos = start + jj;
           const float* value = reinterpret_cast<const float*>(cache) + static_cast<size_t>(pages[key_pos / page_size]) * page_stride +
-                               v_offset + head_offset + static_cast<size_t>(place) * page_size + key_pos % page_size;
+                               v_offset + static_cast<size_t>(place) * page_size + key_pos % page_size;
           const float4 vv = *reinterpret_cast<const float4*>(value);
           const float4 pv = *reinterpret_cast<const float4*>(prob + group * CHUNK + jj);
           acc += pv.x * vv.x;
@@ -139,7 +146,7 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
       }
       for (; jj < last; ++jj) {
         const int key_pos = start + jj;
-        const T* value = cache + static_cast<size_t>(pages[key_pos / page_size]) * page_stride + v_offset + head_offset +
+        const T* value = cache + static_cast<size_t>(pages[key_pos / page_size]) * page_stride + v_offset +
                          static_cast<size_t>(place) * page_size + key_pos % page_size;
         acc += prob[group * CHUNK + jj] * to_float(*value);
       }
@@ -148,20 +155,24 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
   }
   // the groups' results into one, in the order of the groups
   if (place == 0) group_stat[2 * group] = running_max, group_stat[2 * group + 1] = running_sum;
-  if (place < d) group_out[group * d + place] = acc;
+  if (place < dv) group_out[group * dv + place] = acc;
   __syncthreads();
-  if (threadIdx.x < d) {
+  if (threadIdx.x < dv) {
     float top = -INFINITY;
     for (int g = 0; g < kGroups; ++g) top = fmaxf(top, group_stat[2 * g]);
     float total = 0.f, result = 0.f;
+    if (sink != nullptr) {                         // the sink counts once: exp(sink) in the denominator, nothing in the sum of values
+      top = fmaxf(top, sink[h]);
+      total = expf(sink[h] - top);
+    }
     for (int g = 0; g < kGroups; ++g) {
       const float m = group_stat[2 * g];
       if (m == -INFINITY) continue;                // a group that saw no key
       const float w = expf(m - top);
       total += w * group_stat[2 * g + 1];
-      result += w * group_out[g * d + threadIdx.x];
+      result += w * group_out[g * dv + threadIdx.x];
     }
-    out[(static_cast<size_t>(t) * nq + h) * d + threadIdx.x] = from_float<T>(result / total);
+    out[(static_cast<size_t>(t) * nq + h) * dv + threadIdx.x] = from_float<T>(result / total);
   }
 }
 
@@ -176,32 +187,32 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
 // summed in the order of the dims, its maximum and sum are the same reductions over a wave, the
 // values are added in the order of the keys, and the four states meet in the same order at the end.
 // A column therefore gets the same bits from either kernel, and a step may take whichever is faster.
-// Head sizes up to 64.  Tokens of a workgroup that belong to different sequences are served one
+// Head sizes (of keys and of values) up to 64.  Tokens of a workgroup that belong to different sequences are served one
 // run of equal sequences after the other.
 constexpr int kTiledCols = 32, kTiledWaves = 8, kTiledSlots = kTiledCols / kTiledWaves;     // columns a workgroup, its waves, columns a wave
 template <typename T>
 __global__ void __launch_bounds__(64 * kTiledWaves)
 attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
                                int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
-                               T* __restrict__ out, int tokens, int nq, int nkv, int d, int page_size, int window, float scale,
-                               int tokens_per_block, int heads_per_block, const int* __restrict__ seq_start, int min_tokens) {
+                               T* __restrict__ out, int tokens, int nq, int nkv, int d, int dv, int page_size, int window,
+                               int chunk, const float* __restrict__ sink, float scale, int tokens_per_block, int heads_per_block, const int* __restrict__ seq_start, int min_tokens) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // rows of a multiple of 4 floats, so that four values are one LDS read, plus 4: a wave's lanes, each
   // on a row of its own, then spread over the banks
   const int k_stride = (d + 3) / 4 * 4 + 4, q_stride = (d + 3) / 4 * 4;
   constexpr int kValueStride = 68;
   float* k_tile = lds;                             // [64 keys][k_stride]
-  float* v_tile = k_tile + 64 * k_stride;          // [d][68]
-  float* q_tile = v_tile + d * kValueStride;       // [32 columns][q_stride]
+  float* v_tile = k_tile + 64 * k_stride;          // [dv][68]
+  float* q_tile = v_tile + dv * kValueStride;       // [32 columns][q_stride]
   float* prob = q_tile + kTiledCols * q_stride;    // [waves][4 columns][64 keys]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int G = nq / nkv, kv_head = blockIdx.y;
   const int tok0 = blockIdx.x * tokens_per_block, head0 = blockIdx.z * heads_per_block;
   const int ntok = min(tokens_per_block, tokens - tok0), nheads = min(heads_per_block, G - head0);
   const int ncols = ntok * nheads;                 // column c = (token c / nheads, head c % nheads)
-  const size_t page_stride = static_cast<size_t>(2) * nkv * page_size * d;
+  const size_t page_stride = static_cast<size_t>(nkv) * page_size * (d + dv);
   const size_t head_offset = static_cast<size_t>(kv_head) * page_size * d;
-  const size_t v_offset = static_cast<size_t>(nkv) * page_size * d;
+  const size_t v_offset = static_cast<size_t>(nkv) * page_size * d + static_cast<size_t>(kv_head) * page_size * dv;
 
   for (int e = threadIdx.x; e < ncols * d; e += 64 * kTiledWaves) {
     const int c = e / d, i = e - c * d;
@@ -220,6 +231,7 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
     col_tok[s] = live ? c / nheads : -1;
     col_pos[s] = live ? positions[tok0 + col_tok[s]] : -1;
     col_lo[s] = live && window > 0 ? max(0, col_pos[s] - window + 1) : 0;
+    if (live && chunk > 0) col_lo[s] = max(col_lo[s], col_pos[s] - col_pos[s] % chunk);
   }
   float run_max[4][kTiledSlots], run_sum[4][kTiledSlots], acc[4][kTiledSlots];
 #pragma unroll
@@ -244,7 +256,9 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
     for (int t = run_first; t < run_end; ++t) {
       const int pos = positions[tok0 + t];
       hi = max(hi, pos);
-      lo = min(lo, window > 0 ? max(0, pos - window + 1) : 0);
+      int bound = window > 0 ? max(0, pos - window + 1) : 0;
+      if (chunk > 0) bound = max(bound, pos - pos % chunk);
+      lo = min(lo, bound);
     }
     const int* pages = block_table + static_cast<size_t>(seq) * max_blocks;
     for (int base = (lo / 256) * 256; base <= hi; base += 256) {
@@ -259,10 +273,10 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
             k_tile[r * k_stride + i] = to_float(cache[static_cast<size_t>(pages[j / page_size]) * page_stride + head_offset +
                                                       static_cast<size_t>(j % page_size) * d + i]);
         }
-        for (int e = threadIdx.x; e < 64 * d; e += 64 * kTiledWaves) {
+        for (int e = threadIdx.x; e < 64 * dv; e += 64 * kTiledWaves) {
           const int dim = e >> 6, r = e & 63, j = start + r;
           if (j <= hi && j >= lo)
-            v_tile[dim * kValueStride + r] = to_float(cache[static_cast<size_t>(pages[j / page_size]) * page_stride + v_offset + head_offset +
+            v_tile[dim * kValueStride + r] = to_float(cache[static_cast<size_t>(pages[j / page_size]) * page_stride + v_offset +
                                                   static_cast<size_t>(dim) * page_size + j % page_size]);
         }
         __syncthreads();
@@ -323,7 +337,7 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
           __builtin_amdgcn_wave_barrier();
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-          if (lane < d) {
+          if (lane < dv) {
             const float* value = v_tile + lane * kValueStride;
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
@@ -353,7 +367,7 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
     run_first = run_end;
   }
   // the four states of a column into one, in their order
-  if (lane < d) {
+  if (lane < dv) {
 #pragma unroll
     for (int s = 0; s < kTiledSlots; ++s) {
       const int c = wave + kTiledWaves * s;
@@ -362,6 +376,11 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
 #pragma unroll
       for (int g = 0; g < 4; ++g) top = fmaxf(top, run_max[g][s]);
       float total = 0.f, result = 0.f;
+      if (sink != nullptr) {
+        const float own = sink[kv_head * G + head0 + c % nheads];
+        top = fmaxf(top, own);
+        total = expf(own - top);
+      }
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const float m = run_max[g][s];
@@ -370,7 +389,7 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
         total += w * run_sum[g][s];
         result += w * acc[g][s];
       }
-      out[(static_cast<size_t>(tok0 + c / nheads) * nq + kv_head * G + head0 + c % nheads) * d + lane] = from_float<T>(result / total);
+      out[(static_cast<size_t>(tok0 + c / nheads) * nq + kv_head * G + head0 + c % nheads) * dv + lane] = from_float<T>(result / total);
     }
   }
 }
@@ -381,17 +400,20 @@ using namespace tlie;
 
 extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtype, const int* block_table,
                                       int max_blocks, const int* token_seq, const int* positions, void* out,
-                                      int tokens, int nq, int nkv, int d, int page_size, int window, float scale,
-                                      int tiled, const int* seq_start, int min_tokens, void* stream) {
+                                      int tokens, int nq, int nkv, int d, int dv, int page_size, int window, int chunk,
+                                      const float* sink, float scale, int tiled, const int* seq_start, int min_tokens,
+                                      void* stream) {
   // tiled 0: the kernel of one (token, head) a workgroup; 1: the kernel that shares keys among a
   // sequence's tokens (head sizes up to 64); 2: both, each token served by one of them: the second
   // takes the sequences that bring min_tokens tokens or more (seq_start: int32 [sequences + 1], the
   // step's cumulative token counts), the first the others.  A token gets the same bits from either.
-  if (tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 256 || page_size <= 0 || max_blocks <= 0)
+  // (d only bounds the length of a dot product; dv is served by one thread a dim of a group of at most 256)
+  if (tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 4096 || dv <= 0 || dv > 256 || page_size <= 0 ||
+      max_blocks <= 0 || chunk < 0)
     return kBadArgument;
   if (tiled < 0 || tiled > 2 || (tiled == 2 && (seq_start == nullptr || min_tokens < 1))) return kBadArgument;
   if (dtype != kF32 && dtype != kBF16) return kBadArgument;
-  if (d > 64) tiled = 0;
+  if (d > 64 || dv > 64) tiled = 0;
   const int* select = tiled == 2 ? seq_start : nullptr;
   if (tiled) {
     // (the same bits as the kernel below, for steps whose sequences bring several tokens each)
@@ -400,30 +422,34 @@ extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtyp
     const int tokens_per_block = kTiledCols / heads_per_block;
     const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block, nkv, (G + heads_per_block - 1) / heads_per_block);
     const size_t rounded = (static_cast<size_t>(d) + 3) / 4 * 4;
-    const size_t bytes = (64 * (rounded + 4) + static_cast<size_t>(d) * 68 + kTiledCols * rounded + kTiledWaves * 4 * 64) * sizeof(float);
+    const size_t bytes = (64 * (rounded + 4) + static_cast<size_t>(dv) * 68 + kTiledCols * rounded + kTiledWaves * 4 * 64) * sizeof(float);
     if (dtype == kF32)
       hipLaunchKernelGGL((attention_generic_tiled_kernel<float>), grid, dim3(64 * kTiledWaves), bytes, (hipStream_t)stream, (const float*)q,
-                         (const float*)cache, block_table, max_blocks, token_seq, positions, (float*)out, tokens, nq, nkv, d,
-                         page_size, window, scale, tokens_per_block, heads_per_block, select, min_tokens);
+                         (const float*)cache, block_table, max_blocks, token_seq, positions, (float*)out, tokens, nq, nkv, d, dv,
+                         page_size, window, chunk, sink, scale, tokens_per_block, heads_per_block, select, min_tokens);
     else
       hipLaunchKernelGGL((attention_generic_tiled_kernel<bf16>), grid, dim3(64 * kTiledWaves), bytes, (hipStream_t)stream, (const bf16*)q,
-                         (const bf16*)cache, block_table, max_blocks, token_seq, positions, (bf16*)out, tokens, nq, nkv, d,
-                         page_size, window, scale, tokens_per_block, heads_per_block, select, min_tokens);
+                         (const bf16*)cache, block_table, max_blocks, token_seq, positions, (bf16*)out, tokens, nq, nkv, d, dv,
+                         page_size, window, chunk, sink, scale, tokens_per_block, heads_per_block, select, min_tokens);
     const int status = launch_status();
     if (status != kOk || tiled == 1) return status;
   }
-  const int chunk = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
-  const int groups = 256 / chunk;
-  const size_t lds = (static_cast<size_t>(d) + 256 + 4 + 2 * groups + static_cast<size_t>(groups) * d) * sizeof(float);
+  // keys a group of threads takes in one turn: the least of 64, 128, 256 that holds both head sizes (beyond 256 dims of
+  // a key: 256)
+  const int widest = d > dv ? d : dv;
+  const int keys = widest <= 64 ? 64 : (widest <= 128 ? 128 : 256);
+  const int groups = 256 / keys;
+  const size_t lds = (static_cast<size_t>(d) + 256 + 4 + 2 * groups + static_cast<size_t>(groups) * dv) * sizeof(float);
+  if (lds > 64 * 1024) return kBadArgument;
   hipStream_t s = (hipStream_t)stream;
 #define TLIE_LAUNCH(T, CHUNK)                                                                                         \
   hipLaunchKernelGGL((attention_generic_kernel<T, CHUNK>), dim3(tokens, nq), dim3(256), lds, s, (const T*)q,           \
-                     (const T*)cache, block_table, max_blocks, token_seq, positions, (T*)out, nq, nkv, d, page_size,   \
-                     window, scale, select, min_tokens)
+                     (const T*)cache, block_table, max_blocks, token_seq, positions, (T*)out, nq, nkv, d, dv, page_size, \
+                     window, chunk, sink, scale, select, min_tokens)
   if (dtype == kF32) {
-    if (chunk == 64) TLIE_LAUNCH(float, 64); else if (chunk == 128) TLIE_LAUNCH(float, 128); else TLIE_LAUNCH(float, 256);
+    if (keys == 64) TLIE_LAUNCH(float, 64); else if (keys == 128) TLIE_LAUNCH(float, 128); else TLIE_LAUNCH(float, 256);
   } else if (dtype == kBF16) {
-    if (chunk == 64) TLIE_LAUNCH(bf16, 64); else if (chunk == 128) TLIE_LAUNCH(bf16, 128); else TLIE_LAUNCH(bf16, 256);
+    if (keys == 64) TLIE_LAUNCH(bf16, 64); else if (keys == 128) TLIE_LAUNCH(bf16, 128); else TLIE_LAUNCH(bf16, 256);
   }
   else
     return kBadArgument;

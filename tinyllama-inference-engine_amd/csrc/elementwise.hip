@@ -98,12 +98,23 @@ __global__ void add_rmsnorm_wide_kernel(float* __restrict__ residual, const D* _
   }
 }
 
+// ---- the gate of a gated feed-forward, from a gate g and an up u (both float) -------------------------
+// kind 0: silu(g) * u (reference: (g / (1 + exp(-g))) * u in float, src/cuda/kernels.cu:198-206).
+// kind 1: g and u clamped first, g from above only (g = min(g, limit), u in [-limit, limit]), then
+//         g * sigmoid(alpha * g) * (u + 1).
+__device__ __forceinline__ float gated_value(float g, float u, int kind, float alpha, float limit) {
+  if (kind == 0) return (g / (1.f + expf(-g))) * u;
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return (g / (1.f + expf(-alpha * g))) * (u + 1.f);
+}
+
 // ---- act[t, i] = silu(gate[t, i]) * up[t, i]; gate_up is [rows, 2 * inter], either [gate | up] or,
 // interleaved, g0 u0 g1 u1 ... (the layout the gated product of few rows wants of its weight) -------
 // reference: (g / (1 + exp(-g))) * u in float (src/cuda/kernels.cu:198-206)
 template <typename D, typename O>
 __global__ void silu_mul_kernel(const D* __restrict__ gate_up, int nsplit, size_t split_stride,
-                                O* __restrict__ out, int rows, int inter, int interleaved) {
+                                O* __restrict__ out, int rows, int inter, int interleaved, int kind, float alpha, float limit) {
   const size_t total = static_cast<size_t>(rows) * inter;
   for (size_t index = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; index < total;
        index += static_cast<size_t>(gridDim.x) * blockDim.x) {
@@ -111,7 +122,7 @@ __global__ void silu_mul_kernel(const D* __restrict__ gate_up, int nsplit, size_
     const D* base = gate_up + t * 2 * inter;
     const float g = sum_splits(base + (interleaved ? 2 * i : i), nsplit, split_stride);
     const float u = sum_splits(base + (interleaved ? 2 * i + 1 : inter + i), nsplit, split_stride);
-    out[index] = from_float<O>((g / (1.f + expf(-g))) * u);
+    out[index] = from_float<O>(gated_value(g, u, kind, alpha, limit));
   }
 }
 
@@ -119,7 +130,7 @@ __global__ void silu_mul_kernel(const D* __restrict__ gate_up, int nsplit, size_
 // added in the order of their index.
 template <typename D, typename O>
 __global__ void silu_mul_wide_kernel(const D* __restrict__ gate_up, int nsplit, size_t split_stride, O* __restrict__ out,
-                                     int rows, int inter, int interleaved) {
+                                     int rows, int inter, int interleaved, int kind, float alpha, float limit) {
   const int per_row = inter / 8;
   const size_t total = static_cast<size_t>(rows) * per_row;
   for (size_t index = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; index < total;
@@ -151,9 +162,44 @@ __global__ void silu_mul_wide_kernel(const D* __restrict__ gate_up, int nsplit, 
       for (int j = 0; j < 8; ++j) g[j] = a[j], u[j] = b[j];
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) g[j] = (g[j] / (1.f + expf(-g[j]))) * u[j];
+    for (int j = 0; j < 8; ++j) g[j] = gated_value(g[j], u[j], kind, alpha, limit);
     store8(out + t * inter + i, g);
   }
+}
+
+// ---- residual += RMSNorm(delta) * post_weight; out = RMSNorm(residual) * weight ---------------------
+// For blocks that norm a sublayer's result before it joins the residual, and norm the residual again
+// before the next sublayer: both in one pass over the row.  Sums of squares, scales and the residual
+// sum are float.  rows != nullptr: only those rows, and the residual is left as it was; out may be
+// null (the residual is brought up to date and nothing else).
+template <typename D, typename W, typename O>
+__global__ void norm_add_rmsnorm_kernel(float* __restrict__ residual, const D* __restrict__ delta, int nsplit,
+                                        size_t split_stride, const W* __restrict__ post_weight, float post_eps,
+                                        const W* __restrict__ weight, float eps, O* __restrict__ out,
+                                        const int* __restrict__ rows, int hidden) {
+  extern __shared__ float row_cache[];           // hidden floats, then 16 for the reductions
+  float* scratch = row_cache + hidden;
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float* res = residual + static_cast<size_t>(src) * hidden;
+  float square = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = sum_splits(delta + static_cast<size_t>(src) * hidden + i, nsplit, split_stride);
+    row_cache[i] = v;                            // (a thread reads back only what it wrote itself)
+    square += v * v;
+  }
+  const float post_scale = rsqrtf(block_sum(square, scratch) / static_cast<float>(hidden) + post_eps);
+  square = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = res[i] + row_cache[i] * post_scale * to_float(post_weight[i]);
+    if (!rows) res[i] = v;
+    row_cache[i] = v;
+    square += v * v;
+  }
+  if (out == nullptr) return;                    // (the same for the whole grid)
+  const float scale = rsqrtf(block_sum(square, scratch) / static_cast<float>(hidden) + eps);
+  O* o = out + static_cast<size_t>(r) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_float<O>(row_cache[i] * scale * to_float(weight[i]));
 }
 
 // ---- out[r, c] = product[r, c] + bias[c] ------------------------------------------------------
@@ -229,9 +275,38 @@ extern "C" int tlie_add_rmsnorm(float* residual, const void* delta, int delta_dt
   return kBadArgument;
 }
 
+// delta [nsplit][rows][hidden]; post_weight and weight [hidden] of one type; weight and out may be null
+// together (no norm after the add); rows may be null (all rows, residual updated in place).
+extern "C" int tlie_norm_add_rmsnorm(float* residual, const void* delta, int delta_dtype, int nsplit, long long split_stride,
+                                     const void* post_weight, float post_eps, const void* weight, int weight_dtype, float eps,
+                                     void* out, int out_dtype, const int* rows, int num_rows, int hidden, void* stream) {
+  if (num_rows <= 0 || hidden <= 0 || nsplit < 1 || delta == nullptr || post_weight == nullptr) return kBadArgument;
+  if ((out == nullptr) != (weight == nullptr)) return kBadArgument;
+  const size_t lds = (static_cast<size_t>(hidden) + 16) * sizeof(float);
+  if (lds > 160 * 1024) return kBadArgument;
+  const int threads = hidden >= 4096 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 256 : 64));
+  hipStream_t s = (hipStream_t)stream;
+#define TLIE_CASE(DC, D, WC, W, OC, O)                                                                              \
+  if (delta_dtype == DC && weight_dtype == WC && out_dtype == OC) {                                                 \
+    hipLaunchKernelGGL((norm_add_rmsnorm_kernel<D, W, O>), dim3(num_rows), dim3(threads), lds, s, residual,          \
+                       (const D*)delta, nsplit, (size_t)split_stride, (const W*)post_weight, post_eps,              \
+                       (const W*)weight, eps, (O*)out, rows, hidden);                                                \
+    return launch_status();                                                                                         \
+  }
+  TLIE_CASE(kF32, float, kF32, float, kF32, float)
+  TLIE_CASE(kF32, float, kF32, float, kBF16, bf16)
+  TLIE_CASE(kBF16, bf16, kF32, float, kBF16, bf16)
+  TLIE_CASE(kF32, float, kBF16, bf16, kBF16, bf16)
+  TLIE_CASE(kBF16, bf16, kBF16, bf16, kBF16, bf16)
+  TLIE_CASE(kF32, float, kBF16, bf16, kF32, float)
+#undef TLIE_CASE
+  return kBadArgument;
+}
+
 extern "C" int tlie_silu_mul(const void* gate_up, int in_dtype, int nsplit, long long split_stride, void* out,
-                             int out_dtype, int rows, int inter, int interleaved, void* stream) {
-  if (rows <= 0 || inter <= 0 || nsplit < 1) return kBadArgument;
+                             int out_dtype, int rows, int inter, int interleaved, int kind, float alpha, float limit,
+                             void* stream) {
+  if (rows <= 0 || inter <= 0 || nsplit < 1 || kind < 0 || kind > 1) return kBadArgument;
   const size_t total = static_cast<size_t>(rows) * inter;
   const int threads = 256;
   const int blocks = static_cast<int>(total / threads + 1 < 65536 ? total / threads + 1 : 65536);
@@ -242,26 +317,26 @@ extern "C" int tlie_silu_mul(const void* gate_up, int in_dtype, int nsplit, long
     const int wide = static_cast<int>(groups / threads + 1 < 65536 ? groups / threads + 1 : 65536);
     if (in_dtype == kF32 && out_dtype == kF32)
       hipLaunchKernelGGL((silu_mul_wide_kernel<float, float>), dim3(wide), dim3(threads), 0, s, (const float*)gate_up,
-                         nsplit, (size_t)split_stride, (float*)out, rows, inter, interleaved);
+                         nsplit, (size_t)split_stride, (float*)out, rows, inter, interleaved, kind, alpha, limit);
     else if (in_dtype == kF32 && out_dtype == kBF16)
       hipLaunchKernelGGL((silu_mul_wide_kernel<float, bf16>), dim3(wide), dim3(threads), 0, s, (const float*)gate_up,
-                         nsplit, (size_t)split_stride, (bf16*)out, rows, inter, interleaved);
+                         nsplit, (size_t)split_stride, (bf16*)out, rows, inter, interleaved, kind, alpha, limit);
     else if (in_dtype == kBF16 && out_dtype == kBF16)
       hipLaunchKernelGGL((silu_mul_wide_kernel<bf16, bf16>), dim3(wide), dim3(threads), 0, s, (const bf16*)gate_up,
-                         nsplit, (size_t)split_stride, (bf16*)out, rows, inter, interleaved);
+                         nsplit, (size_t)split_stride, (bf16*)out, rows, inter, interleaved, kind, alpha, limit);
     else
       return kBadArgument;
     return launch_status();
   }
   if (in_dtype == kF32 && out_dtype == kF32)
     hipLaunchKernelGGL((silu_mul_kernel<float, float>), dim3(blocks), dim3(threads), 0, s, (const float*)gate_up, nsplit,
-                       (size_t)split_stride, (float*)out, rows, inter, interleaved);
+                       (size_t)split_stride, (float*)out, rows, inter, interleaved, kind, alpha, limit);
   else if (in_dtype == kF32 && out_dtype == kBF16)
     hipLaunchKernelGGL((silu_mul_kernel<float, bf16>), dim3(blocks), dim3(threads), 0, s, (const float*)gate_up, nsplit,
-                       (size_t)split_stride, (bf16*)out, rows, inter, interleaved);
+                       (size_t)split_stride, (bf16*)out, rows, inter, interleaved, kind, alpha, limit);
   else if (in_dtype == kBF16 && out_dtype == kBF16)
     hipLaunchKernelGGL((silu_mul_kernel<bf16, bf16>), dim3(blocks), dim3(threads), 0, s, (const bf16*)gate_up, nsplit,
-                       (size_t)split_stride, (bf16*)out, rows, inter, interleaved);
+                       (size_t)split_stride, (bf16*)out, rows, inter, interleaved, kind, alpha, limit);
   else
     return kBadArgument;
   return launch_status();

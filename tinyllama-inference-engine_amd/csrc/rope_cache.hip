@@ -139,9 +139,75 @@ __global__ void rope_cache_wide_kernel(const D* __restrict__ qkv, const int* __r
   }
 }
 
+// The same for any sizes: value heads of a size dv of their own (a page then holds nkv planes of keys
+// [row][d] and after them nkv planes of values [dv][row]), or no key and value heads at all (nkv = 0: the
+// layer reads another layer's cache and only its queries are placed).  Columns in natural order; a
+// rotated element reads its partner's summands itself.  One block a token.
+template <typename D, typename A>
+__global__ void qkv_place_kernel(const D* __restrict__ qkv, int nsplit, size_t split_stride,
+                                 const int* __restrict__ positions, const int* __restrict__ slot_map,
+                                 const float* __restrict__ inv_freq, int rot_dim, A* __restrict__ q_out,
+                                 A* __restrict__ cache, int nq, int nkv, int d, int dv, int page_size) {
+  extern __shared__ float lds[];
+  const int half = rot_dim / 2;
+  float* cosines = lds;                  // half
+  float* sines = cosines + half;         // half
+  const int t = blockIdx.x;
+  const int rotated = (nq + nkv) * d, width = rotated + nkv * dv;
+  if (inv_freq != nullptr) {
+    const float pos = static_cast<float>(positions[t]);
+    for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &sines[i], &cosines[i]);
+    __syncthreads();
+  }
+  const int slot = nkv > 0 ? slot_map[t] : -1;
+  A* page = cache + static_cast<size_t>(slot < 0 ? 0 : slot / page_size) * nkv * page_size * (d + dv);
+  const int row = slot < 0 ? 0 : slot % page_size;
+  const D* in = qkv + static_cast<size_t>(t) * width;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    if (c >= nq * d && slot < 0) break;  // (columns only grow: what is left is keys and values too)
+    float v = sum_splits(in + c, nsplit, split_stride);
+    if (c >= rotated) {
+      const int head = (c - rotated) / dv, e = (c - rotated) % dv;
+      page[static_cast<size_t>(nkv) * page_size * d + (static_cast<size_t>(head) * dv + e) * page_size + row] = from_float<A>(v);
+      continue;
+    }
+    const int head = c / d, e = c % d;
+    if (inv_freq != nullptr && e < rot_dim) {
+      if (e < half) v = v * cosines[e] - sum_splits(in + c + half, nsplit, split_stride) * sines[e];
+      else v = v * cosines[e - half] + sum_splits(in + c - half, nsplit, split_stride) * sines[e - half];
+    }
+    if (head < nq) q_out[static_cast<size_t>(t) * nq * d + c] = from_float<A>(v);
+    else page[(static_cast<size_t>(head - nq) * page_size + row) * d + e] = from_float<A>(v);
+  }
+}
+
 }  // namespace tlie
 
 using namespace tlie;
+
+// q heads of d | k heads of d | v heads of dv; see qkv_place_kernel.
+extern "C" int tlie_qkv_place(const void* qkv, int in_dtype, int nsplit, long long split_stride, const int* positions,
+                              const int* slot_map, const float* inv_freq, int rot_dim, void* q_out, void* cache,
+                              int act_dtype, int tokens, int nq, int nkv, int d, int dv, int page_size, void* stream) {
+  if (tokens <= 0 || nq <= 0 || nkv < 0 || d <= 0 || dv <= 0 || page_size <= 0 || nsplit < 1) return kBadArgument;
+  if (rot_dim < 0 || rot_dim > d || rot_dim % 2 != 0 || (nkv > 0 && (cache == nullptr || slot_map == nullptr))) return kBadArgument;
+  const int width = (nq + nkv) * d + nkv * dv;
+  const int threads = width >= 1024 ? 1024 : (width + 63) / 64 * 64;
+  const size_t lds = static_cast<size_t>(rot_dim) * sizeof(float);
+  hipStream_t s = (hipStream_t)stream;
+#define TLIE_CASE(DC, D, AC, A)                                                                                \
+  if (in_dtype == DC && act_dtype == AC) {                                                                     \
+    hipLaunchKernelGGL((qkv_place_kernel<D, A>), dim3(tokens), dim3(threads), lds, s, (const D*)qkv, nsplit,     \
+                       (size_t)split_stride, positions, slot_map, inv_freq, rot_dim, (A*)q_out, (A*)cache, nq,  \
+                       nkv, d, dv, page_size);                                                                 \
+    return launch_status();                                                                                    \
+  }
+  TLIE_CASE(kF32, float, kF32, float)
+  TLIE_CASE(kF32, float, kBF16, bf16)
+  TLIE_CASE(kBF16, bf16, kBF16, bf16)
+#undef TLIE_CASE
+  return kBadArgument;
+}
 
 extern "C" int tlie_rope_cache(const void* qkv, int in_dtype, int nsplit, long long split_stride,
                                const int* positions, const int* slot_map, const float* inv_freq, int rot_dim,

@@ -1,4 +1,4 @@
-from . import llama  # noqa: F401  (registers the architecture)
+from . import fadutar, llama  # noqa: F401  (each registers its architecture)
 from .builder import DecoderModel, build_model, expected_tensors
 
 __all__ = ["DecoderModel", "build_model", "expected_tensors"]

@@ -90,6 +90,15 @@ class Product:
         return out if dtype is None or out.dtype == dtype else out.to(dtype)
 
 
+@dataclass
+class NormedDelta:
+    """A sublayer's result that is normed before it joins the residual: the product, and the weight and
+    eps of that RMS norm.  Whoever norms the residual next does both in one kernel (`norm_add_rmsnorm`)."""
+    product: Product
+    weight: torch.Tensor
+    eps: float
+
+
 def as_product(value) -> Product:
     if isinstance(value, Product):
         return value
@@ -152,26 +161,42 @@ def add_rmsnorm(residual: torch.Tensor, delta: Product | None, weight: torch.Ten
     return out
 
 
-def silu_mul(gate_up: Product, out_dtype: torch.dtype, interleaved: bool = False) -> torch.Tensor:
+GATES = {"silu": 0, "clamped_swish": 1}
+
+
+def silu_mul(gate_up: Product, out_dtype: torch.dtype, interleaved: bool = False, gate: str = "silu", alpha: float = 1.0,
+             limit: float = 0.0) -> torch.Tensor:
     """out[t, i] = silu(gate[t, i]) * up[t, i], with gate_up = [gate | up] side by side or, interleaved,
-    g0 u0 g1 u1 ..."""
+    g0 u0 g1 u1 ...  gate "clamped_swish": g = min(gate, limit), u = clamp(up, -limit, limit),
+    out = g * sigmoid(alpha * g) * (u + 1)."""
     _check_product(gate_up, "gate_up")
+    if gate not in GATES:
+        raise invalid_argument(f"silu_mul: unknown gate '{gate}'")
+    if gate == "clamped_swish" and not limit > 0.0:
+        raise invalid_argument("silu_mul: the clamped gate needs a positive limit")
     if gate_up.cols % 2 != 0:
         raise invalid_shape("silu_mul: the input holds gate and up side by side, its width must be even")
     rows, inter = gate_up.rows, gate_up.cols // 2
     out = torch.empty((rows, inter), dtype=out_dtype, device=gate_up.data.device)
     _check(library().tlie_silu_mul(_ptr(gate_up.data), dtype_code(gate_up.data.dtype), gate_up.nsplit,
                                    ctypes.c_longlong(gate_up.split_stride), _ptr(out), dtype_code(out_dtype), rows, inter,
-                                   1 if interleaved else 0, _stream()), "silu_mul")
+                                   1 if interleaved else 0, GATES[gate], ctypes.c_float(alpha), ctypes.c_float(limit),
+                                   _stream()), "silu_mul")
     return out
 
 
-def _check_cache(cache: torch.Tensor, num_kv_heads: int, head_dim: int, what: str) -> int:
+def _check_cache(cache: torch.Tensor, num_kv_heads: int, head_dim: int, what: str, value_dim: int | None = None) -> int:
     """cache: [pages, 2, nkv, page_size * d]; per page and kv head the keys lie as [row][dim] and
-    the values transposed, [dim][row].  Returns the page size."""
-    if cache.dim() != 4 or cache.shape[1] != 2 or cache.shape[2] != num_kv_heads or cache.shape[3] % head_dim != 0:
-        raise invalid_shape(f"{what}: cache {list(cache.shape)} is not [pages, 2, nkv, page_size * d]")
-    return cache.shape[3] // head_dim
+    the values transposed, [dim][row].  With a value size dv of its own a page is
+    [nkv, page_size * (d + dv)] instead: the nkv planes of keys, then the nkv planes of values
+    (the same order of bytes when dv = d).  Returns the page size."""
+    if value_dim is None or value_dim == head_dim:
+        if cache.dim() != 4 or cache.shape[1] != 2 or cache.shape[2] != num_kv_heads or cache.shape[3] % head_dim != 0:
+            raise invalid_shape(f"{what}: cache {list(cache.shape)} is not [pages, 2, nkv, page_size * d]")
+        return cache.shape[3] // head_dim
+    if cache.dim() != 3 or cache.shape[1] != num_kv_heads or cache.shape[2] % (head_dim + value_dim) != 0:
+        raise invalid_shape(f"{what}: cache {list(cache.shape)} is not [pages, nkv, page_size * (d + dv)]")
+    return cache.shape[2] // (head_dim + value_dim)
 
 
 def paired_rows(num_heads: int, num_kv_heads: int, head_dim: int, rot_dim: int) -> torch.Tensor:
@@ -225,7 +250,8 @@ def rope_cache(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor, in
 def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, token_seq: torch.Tensor,
                       positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                       window: int | None, scale: float, tiled: bool | int = False, seq_start: torch.Tensor | None = None,
-                      min_tokens: int = GENERIC_TILED_MIN_TOKENS) -> torch.Tensor:
+                      min_tokens: int = GENERIC_TILED_MIN_TOKENS, value_dim: int | None = None, chunk: int | None = None,
+                      sink: torch.Tensor | None = None) -> torch.Tensor:
     """Causal attention of every token over its sequence's cached keys; any number of tokens per
     sequence.  block_table: [sequences, max_blocks] pages; token_seq[t]: the token's row of it.
     tiled 1 (True): the step's sequences bring several tokens each (consecutive in the step, at
@@ -233,8 +259,21 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
     64; the result has the same bits either way).  tiled 2: both kernels are launched and every token
     is served by one of them: by the tiled one if its sequence brings `min_tokens` tokens or more
     (seq_start: the step's cumulative token counts [sequences + 1], on the device), by the plain one
-    otherwise: for steps that mix portions of prompts with single tokens."""
+    otherwise: for steps that mix portions of prompts with single tokens.
+    value_dim: the size of a value head when it is not the key heads' (see `_check_cache`); the result is
+    [tokens, nq * value_dim].  chunk: a token sees only the keys of its own chunk of so many positions
+    (counted from position 0).  sink: float32 [nq], a number per head whose exponential joins the
+    softmax's denominator."""
     _device_tensor(q, "q", (torch.float32, torch.bfloat16))
+    value_dim = head_dim if value_dim is None else int(value_dim)
+    if sink is not None:
+        _device_tensor(sink, "sink", torch.float32)
+        if sink.shape != (num_heads,):
+            raise invalid_shape("attention: the sink needs one entry per query head")
+    if chunk is not None and int(chunk) <= 0:
+        raise invalid_argument("attention: a chunk must be a positive count of positions")
+    if not 0 < value_dim <= ATTENTION_MAX_HEAD_DIM:
+        raise invalid_argument(f"attention: the plain kernel takes value heads of 1 to {ATTENTION_MAX_HEAD_DIM} dims")
     _device_tensor(cache, "cache", q.dtype)
     _device_tensor(block_table, "block_table", torch.int32)
     _device_tensor(token_seq, "token_seq", torch.int32)
@@ -242,7 +281,7 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
     tokens = q.shape[0]
     if q.shape != (tokens, num_heads * head_dim):
         raise invalid_shape(f"attention: q {list(q.shape)} is not [tokens, nq * d]")
-    page_size = _check_cache(cache, num_kv_heads, head_dim, "attention")
+    page_size = _check_cache(cache, num_kv_heads, head_dim, "attention", value_dim)
     if block_table.dim() != 2 or token_seq.shape != (tokens,) or positions.shape != (tokens,):
         raise invalid_shape("attention: block_table must be [sequences, max_blocks], token_seq and positions [tokens]")
     if num_heads % num_kv_heads != 0:
@@ -254,24 +293,25 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
             raise invalid_shape("attention: seq_start needs one entry more than the block table has rows, min_tokens at least 1")
     elif tiled not in (0, 1):
         raise invalid_argument("attention: tiled is 0, 1 or 2")
-    out = torch.empty_like(q)
+    out = torch.empty((tokens, num_heads * value_dim), dtype=q.dtype, device=q.device)
     _check(library().tlie_attention_generic(_ptr(q), _ptr(cache), dtype_code(q.dtype), _ptr(block_table),
                                             block_table.shape[1], _ptr(token_seq), _ptr(positions), _ptr(out), tokens,
-                                            num_heads, num_kv_heads, head_dim, page_size,
-                                            int(window) if window else 0, ctypes.c_float(scale), tiled,
+                                            num_heads, num_kv_heads, head_dim, value_dim, page_size,
+                                            int(window) if window else 0, int(chunk) if chunk else 0, _ptr(sink),
+                                            ctypes.c_float(scale), tiled,
                                             _ptr(seq_start if tiled == 2 else None), int(min_tokens), _stream()),
            "attention_generic")
     return out
 
 
-def attention_generic_plan(ctx, head_dim: int) -> int:
+def attention_generic_plan(ctx, head_dim: int, value_dim: int | None = None) -> int:
     """Which form of the plain attention kernel a step takes (the `tiled` of `attention_generic`): the
     one that shares each read of the keys among a sequence's tokens pays from a few tokens a
     sequence on, and costs dearly where a workgroup's 32 columns belong to many sequences of one
     token (it walks each one's context in turn).  A launched step is decided from its host arrays;
     a recorded step of portions, whose cut changes from replay to replay, launches both and lets
     each sequence's token count on the device decide."""
-    if head_dim > 64 or ctx.max_new < GENERIC_TILED_MIN_TOKENS:
+    if max(head_dim, value_dim or head_dim) > 64 or ctx.max_new < GENERIC_TILED_MIN_TOKENS:
         return 0
     if ctx.tile_owner is not None:
         return 2
@@ -279,6 +319,202 @@ def attention_generic_plan(ctx, head_dim: int) -> int:
     counts = starts[1:] - starts[:-1]
     many = int((counts >= GENERIC_TILED_MIN_TOKENS).sum())
     return 1 if many == len(counts) else (2 if many else 0)
+
+
+def norm_add_rmsnorm(residual: torch.Tensor, delta: Product, post_weight: torch.Tensor, post_eps: float,
+                     weight: torch.Tensor | None, eps: float, out_dtype: torch.dtype,
+                     rows: torch.Tensor | None = None) -> torch.Tensor | None:
+    """residual += RMSNorm(delta) * post_weight (all rows, in place), then out = RMSNorm(residual) * weight:
+    a sublayer's result is normed before it joins the residual, and the residual before the next
+    sublayer, in one pass.  weight None: only the residual is brought up to date (returns None).  With
+    `rows` only those rows are computed, and the residual is left as it was."""
+    _device_tensor(residual, "residual", torch.float32)
+    _check_product(delta, "delta")
+    _device_tensor(post_weight, "post norm weight", (torch.float32, torch.bfloat16))
+    tokens, hidden = residual.shape
+    if (delta.rows, delta.cols) != (tokens, hidden) or post_weight.shape != (hidden,):
+        raise invalid_shape(f"norm_add_rmsnorm: delta [{delta.rows}, {delta.cols}] or the weight do not fit residual {list(residual.shape)}")
+    if weight is not None:
+        _device_tensor(weight, "norm weight", post_weight.dtype)
+        if weight.shape != (hidden,):
+            raise invalid_shape("norm_add_rmsnorm: the norm's weight needs one entry per column")
+    if not (post_eps > 0.0 and eps > 0.0):
+        raise EngineError(ErrorCode.NUMERICAL, "RMSNorm requires a positive epsilon")
+    count = tokens
+    if rows is not None:
+        _device_tensor(rows, "rows", torch.int32)
+        count = rows.shape[0]
+    out = torch.empty((count, hidden), dtype=out_dtype, device=residual.device) if weight is not None else None
+    if count == 0:
+        return out
+    _check(library().tlie_norm_add_rmsnorm(_ptr(residual), _ptr(delta.data), dtype_code(delta.data.dtype), delta.nsplit,
+                                           ctypes.c_longlong(delta.split_stride), _ptr(post_weight), ctypes.c_float(post_eps),
+                                           _ptr(weight), dtype_code(post_weight.dtype), ctypes.c_float(eps), _ptr(out),
+                                           dtype_code(out_dtype), _ptr(rows), count, hidden, _stream()), "norm_add_rmsnorm")
+    return out
+
+
+def qkv_place(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor | None, inv_freq: torch.Tensor | None,
+              rot_dim: int, cache: torch.Tensor | None, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+              act_dtype: torch.dtype) -> torch.Tensor:
+    """`rope_cache` for any sizes: value heads of `value_dim` dims (a page is then nkv planes of keys and
+    after them nkv planes of transposed values), and num_kv_heads 0 for a layer that reads another
+    layer's cache: only its queries [T, nq * d] are rotated and returned, nothing is written."""
+    _check_product(qkv, "qkv")
+    _device_tensor(positions, "positions", torch.int32)
+    tokens = qkv.rows
+    if qkv.cols != (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim:
+        raise invalid_shape(f"qkv_place: qkv width {qkv.cols} is not (nq + nkv) * d + nkv * dv")
+    if positions.shape != (tokens,):
+        raise invalid_shape("qkv_place: positions need one entry per token")
+    page_size = 1
+    if num_kv_heads > 0:
+        _device_tensor(slot_map, "slot_map", torch.int32)
+        _device_tensor(cache, "cache", act_dtype)
+        if slot_map.shape != (tokens,):
+            raise invalid_shape("qkv_place: slot_map needs one entry per token")
+        page_size = _check_cache(cache, num_kv_heads, head_dim, "qkv_place", value_dim)
+    if inv_freq is not None:
+        _device_tensor(inv_freq, "inv_freq", torch.float32)
+        if rot_dim % 2 != 0 or not 0 < rot_dim <= head_dim or inv_freq.shape != (rot_dim // 2,):
+            raise invalid_shape("qkv_place: inv_freq needs rot_dim / 2 entries, rot_dim even and at most d")
+    else:
+        rot_dim = 0
+    q_out = torch.empty((tokens, num_heads * head_dim), dtype=act_dtype, device=qkv.data.device)
+    _check(library().tlie_qkv_place(_ptr(qkv.data), dtype_code(qkv.data.dtype), qkv.nsplit, ctypes.c_longlong(qkv.split_stride),
+                                    _ptr(positions), _ptr(slot_map if num_kv_heads > 0 else None), _ptr(inv_freq), rot_dim,
+                                    _ptr(q_out), _ptr(cache if num_kv_heads > 0 else None), dtype_code(act_dtype), tokens,
+                                    num_heads, num_kv_heads, head_dim, value_dim, page_size, _stream()), "qkv_place")
+    return q_out
+
+
+def block_linear(x: torch.Tensor, x_offset: int, x_row: int, x_block: int, weight_t: torch.Tensor, bias: torch.Tensor | None,
+                 out: torch.Tensor, out_offset: int, out_row: int, out_block: int, rows: int) -> None:
+    """Block-diagonal product: for each of weight_t's blocks b, rows of `inner` values that lie in the flat
+    array x at x_offset + row * x_row + b * x_block are multiplied by weight_t[b] ([inner, outer], the
+    block's matrix transposed) and, plus bias[b], written to the flat array `out` at out_offset + row *
+    out_row + b * out_block.  Sums are float."""
+    _device_tensor(x, "x", (torch.float32, torch.bfloat16))
+    _device_tensor(weight_t, "weight", (torch.float32, torch.bfloat16))
+    _device_tensor(out, "out", (torch.float32, torch.bfloat16))
+    if weight_t.dim() != 3:
+        raise invalid_shape("block_linear: the weight must be [blocks, inner, outer]")
+    blocks, inner, outer = weight_t.shape
+    if bias is not None:
+        _device_tensor(bias, "bias", weight_t.dtype)
+        if bias.shape != (blocks, outer):
+            raise invalid_shape("block_linear: the bias must be [blocks, outer]")
+    if rows <= 0:
+        return
+    if min(x_offset, x_row, x_block, out_offset, out_row, out_block) < 0:
+        raise invalid_argument("block_linear: offsets and strides must not be negative")
+    if x_offset + (rows - 1) * x_row + (blocks - 1) * x_block + inner > x.numel():
+        raise invalid_shape("block_linear: the strides reach beyond x")
+    if out_offset + (rows - 1) * out_row + (blocks - 1) * out_block + outer > out.numel():
+        raise invalid_shape("block_linear: the strides reach beyond out")
+    x_address = x.data_ptr() + x_offset * x.element_size()
+    out_address = out.data_ptr() + out_offset * out.element_size()
+    _check(library().tlie_block_linear(ctypes.c_void_p(x_address), dtype_code(x.dtype), ctypes.c_longlong(x_row),
+                                       ctypes.c_longlong(x_block), _ptr(weight_t), dtype_code(weight_t.dtype), _ptr(bias),
+                                       ctypes.c_void_p(out_address), dtype_code(out.dtype), ctypes.c_longlong(out_row),
+                                       ctypes.c_longlong(out_block), rows, blocks, inner, outer, _stream()), "block_linear")
+
+
+def latent_place(fused: Product, positions: torch.Tensor, slot_map: torch.Tensor, inv_freq: torch.Tensor | None,
+                 norm_weight: torch.Tensor, eps: float, cache: torch.Tensor, heads: int, plain: int, rot: int, rank: int,
+                 act_dtype: torch.dtype) -> tuple[torch.Tensor, torch.Tensor]:
+    """Latent attention between its first product and the attention kernel.  fused: [T, heads * (plain +
+    rot) + rank + rot].  The rank dims are RMS-normed (weight, eps) and written to the cache rows of
+    `slot_map` as keys [row][rank + rot] beside the rotated shared key part, and once more, transposed, as
+    values; returns (q_plain [T, heads * plain], q_wide [T, heads, rank + rot] of which only each head's
+    last rot dims, the rotated ones, are filled: the per-head product of q_plain fills the rest)."""
+    _check_product(fused, "fused")
+    _device_tensor(positions, "positions", torch.int32)
+    _device_tensor(slot_map, "slot_map", torch.int32)
+    _device_tensor(cache, "cache", act_dtype)
+    _device_tensor(norm_weight, "latent norm weight", (torch.float32, torch.bfloat16))
+    tokens = fused.rows
+    if fused.cols != heads * (plain + rot) + rank + rot or norm_weight.shape != (rank,):
+        raise invalid_shape(f"latent_place: width {fused.cols} is not heads * (plain + rot) + rank + rot")
+    if positions.shape != (tokens,) or slot_map.shape != (tokens,):
+        raise invalid_shape("latent_place: positions and slot_map need one entry per token")
+    if rot % 2 != 0 or rot < 0 or (rot > 0 and (inv_freq is None or inv_freq.shape != (rot // 2,))):
+        raise invalid_shape("latent_place: inv_freq needs rot / 2 entries, rot even")
+    if inv_freq is not None:
+        _device_tensor(inv_freq, "inv_freq", torch.float32)
+    if not eps > 0.0:
+        raise EngineError(ErrorCode.NUMERICAL, "RMSNorm requires a positive epsilon")
+    page_size = _check_cache(cache, 1, rank + rot, "latent_place", rank)
+    q_plain = torch.empty((tokens, heads * plain), dtype=act_dtype, device=cache.device)
+    q_wide = torch.empty((tokens, heads * (rank + rot)), dtype=act_dtype, device=cache.device)
+    _check(library().tlie_latent_place(_ptr(fused.data), dtype_code(fused.data.dtype), fused.nsplit,
+                                       ctypes.c_longlong(fused.split_stride), _ptr(positions), _ptr(slot_map), _ptr(inv_freq),
+                                       _ptr(norm_weight), dtype_code(norm_weight.dtype), ctypes.c_float(eps), _ptr(q_plain),
+                                       _ptr(q_wide), _ptr(cache), dtype_code(act_dtype), tokens, heads, plain, rot, rank,
+                                       page_size, _stream()), "latent_place")
+    return q_plain, q_wide
+
+
+def causal_conv(fused: Product, x_col: int, taps: torch.Tensor, bias: torch.Tensor | None, state: torch.Tensor,
+                token_seq: torch.Tensor, token_slot: torch.Tensor, seq_start: torch.Tensor) -> torch.Tensor:
+    """A causal convolution per channel over each sequence's tokens of the step: columns x_col .. x_col +
+    channels - 1 of `fused` are its inputs, taps [channels, n] (the last tap is the current token's), what came
+    before the step is read from state [slots, n, channels] (rows 0 .. n-2: the last inputs, oldest first).
+    Returns float32 [T, channels]; rows of tokens whose slot is negative are left unwritten."""
+    _check_product(fused, "fused")
+    _device_tensor(taps, "taps", (torch.float32, torch.bfloat16))
+    _device_tensor(state, "state", torch.float32)
+    for name, tensor in (("token_seq", token_seq), ("token_slot", token_slot), ("seq_start", seq_start)):
+        _device_tensor(tensor, name, torch.int32)
+    if taps.dim() != 2:
+        raise invalid_shape("causal_conv: taps must be [channels, n]")
+    channels, count = taps.shape
+    tokens = fused.rows
+    if bias is not None:
+        _device_tensor(bias, "bias", taps.dtype)
+        if bias.shape != (channels,):
+            raise invalid_shape("causal_conv: the bias needs one entry per channel")
+    if state.dim() != 3 or state.shape[1:] != (count, channels) or not 0 <= x_col <= fused.cols - channels:
+        raise invalid_shape(f"causal_conv: state {list(state.shape)} is not [slots, {count}, {channels}], or the columns do not fit")
+    if token_seq.shape != (tokens,) or token_slot.shape != (tokens,) or seq_start.dim() != 1:
+        raise invalid_shape("causal_conv: token_seq and token_slot need one entry per token")
+    u = torch.empty((tokens, channels), dtype=torch.float32, device=state.device)
+    _check(library().tlie_causal_conv(_ptr(fused.data), dtype_code(fused.data.dtype), fused.nsplit,
+                                      ctypes.c_longlong(fused.split_stride), fused.cols, x_col, _ptr(taps), _ptr(bias),
+                                      dtype_code(taps.dtype), _ptr(state), _ptr(token_seq), _ptr(token_slot), _ptr(seq_start),
+                                      _ptr(u), tokens, channels, count, _stream()), "causal_conv")
+    return u
+
+
+def gated_recurrence(fused: Product, x_col: int, y_col: int, u: torch.Tensor, gates: torch.Tensor, lam: torch.Tensor,
+                     decay: float, state: torch.Tensor, seq_start: torch.Tensor, seq_slot: torch.Tensor, block_width: int,
+                     out_dtype: torch.dtype) -> torch.Tensor:
+    """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t with a_t = exp(-decay * r_t * softplus(lam)), r and i the
+    sigmoids of `gates` [T, blocks, 2 * block_width] (a block's r before its i), per channel and sequence,
+    from and to row n-1 of state [slots, n, channels]; out = S * gelu_tanh(y), y in columns y_col .. of
+    `fused`; the state's other rows get the step's last inputs of the convolution (columns x_col ..).
+    Sequences whose slot is negative are skipped."""
+    _check_product(fused, "fused")
+    _device_tensor(u, "u", torch.float32)
+    _device_tensor(gates, "gates", torch.float32)
+    _device_tensor(lam, "lambda", (torch.float32, torch.bfloat16))
+    _device_tensor(state, "state", torch.float32)
+    _device_tensor(seq_start, "seq_start", torch.int32)
+    _device_tensor(seq_slot, "seq_slot", torch.int32)
+    tokens, channels = u.shape
+    seqs = seq_slot.shape[0]
+    if (fused.rows != tokens or gates.numel() != tokens * 2 * channels or lam.shape != (channels,) or state.dim() != 3
+            or state.shape[2] != channels or seq_start.shape != (seqs + 1,) or block_width <= 0 or channels % block_width != 0):
+        raise invalid_shape("gated_recurrence: the operands do not fit each other")
+    if not (0 <= x_col <= fused.cols - channels and 0 <= y_col <= fused.cols - channels):
+        raise invalid_shape("gated_recurrence: the columns do not fit the product")
+    out = torch.empty((tokens, channels), dtype=out_dtype, device=u.device)
+    _check(library().tlie_gated_recurrence(_ptr(fused.data), dtype_code(fused.data.dtype), fused.nsplit,
+                                           ctypes.c_longlong(fused.split_stride), fused.cols, x_col, y_col, _ptr(u), _ptr(gates),
+                                           _ptr(lam), dtype_code(lam.dtype), ctypes.c_float(decay), _ptr(state), _ptr(seq_start),
+                                           _ptr(seq_slot), _ptr(out), dtype_code(out_dtype), seqs, channels, block_width,
+                                           state.shape[1], _stream()), "gated_recurrence")
+    return out
 
 
 def gemm_generic(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out_dtype: torch.dtype) -> Product:

@@ -1,4 +1,4 @@
-from . import attention, block, embedding, mlp, norm, rotary  # noqa: F401  (each registers its parts)
+from . import attention, block, embedding, latent_attention, mlp, norm, recurrent, rotary  # noqa: F401  (each registers its parts)
 from .base import Binding, FeedForward, CacheNeed, Mixer, Norm, Part, PositionEncoding, StateNeed
 from .linear import Linear
 

@@ -26,8 +26,19 @@ from .linear import Linear
 @register("mixer", "attention")
 class Attention(Mixer):
     """spec: hidden_size, num_heads, num_kv_heads, head_dim, bias, window (None or a count of
-    positions), position (a PartSpec of a position encoding).
-    Tensors: `<prefix>{q,k,v,o}_proj.weight` (and `.bias` when bias)."""
+    positions), position (a PartSpec of a position encoding).  Optionally:
+      value_dim          the size of a value head (default head_dim)
+      scale              of the scores (default 1 / sqrt(head_dim))
+      chunk              a token sees only the keys of its own chunk of so many positions, counted from 0
+      sink               a learned number per head whose exponential joins the softmax's denominator
+      reads_other_cache  the layer has no key and value projections: it reads the cache its run names
+      cache_window       how long the cache keeps a position (default: window, or chunk); the owner of a
+                         cache that other layers read names the longest reach among them (None: for good)
+      names              the tensors' names after the prefix, by role (q, k, v, o, q_bias .. o_bias, sink)
+    Tensors: `<prefix>{q,k,v,o}_proj.weight` (and `.bias` when bias) unless `names` says otherwise."""
+    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+             "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
+             "sink": "sinks"}
 
     def __init__(self, spec: PartSpec, dtype, device):
         super().__init__(spec, dtype, device)
@@ -47,34 +58,60 @@ class Attention(Mixer):
             raise invalid_config("attention: a window must be a positive count of positions")
         position = spec.get("position") or PartSpec("none")
         self.position = lookup("position_encoding", position.kind)(position, dtype, device)
-        self.scale = 1.0 / math.sqrt(float(self.d))
-        self.qkv = self.o = None
+        self.dv = int(spec.get("value_dim") or self.d)
+        self.scale = float(spec["scale"]) if spec.get("scale") is not None else 1.0 / math.sqrt(float(self.d))
+        self.chunk = spec.get("chunk")
+        self.has_sink = bool(spec.get("sink", False))
+        self.reads_other_cache = bool(spec.get("reads_other_cache", False))
+        if not 0 < self.dv <= ops.ATTENTION_MAX_HEAD_DIM:
+            raise invalid_config(f"attention: value_dim {self.dv} is beyond what the attention kernels take")
+        if self.chunk is not None and int(self.chunk) <= 0:
+            raise invalid_config("attention: a chunk must be a positive count of positions")
+        if not (self.scale > 0.0 and math.isfinite(self.scale)):
+            raise invalid_config("attention: the scale of the scores must be positive")
+        # what the kernels that are fused for the plain case (one head size, no sink, no chunks, own keys
+        # and values) do not take goes through the kernels for any sizes
+        self.general = self.dv != self.d or self.has_sink or self.chunk is not None or self.reads_other_cache
+        self.names = {**self.NAMES, **dict(spec.get("names") or {})}
+        self.qkv = self.o = self.sink = None
 
     @classmethod
     def tensor_specs(cls, spec, prefix):
+        names = {**cls.NAMES, **dict(spec.get("names") or {})}
         hidden, d = int(spec["hidden_size"]), int(spec["head_dim"])
-        qd, kvd = int(spec["num_heads"]) * d, int(spec["num_kv_heads"]) * d
-        shapes = (("q_proj", (qd, hidden)), ("k_proj", (kvd, hidden)), ("v_proj", (kvd, hidden)), ("o_proj", (hidden, qd)))
-        specs = [TensorSpec(f"{prefix}{name}.weight", shape) for name, shape in shapes]
+        dv = int(spec.get("value_dim") or d)
+        nq, nkv = int(spec["num_heads"]), int(spec["num_kv_heads"])
+        shapes = [("q", (nq * d, hidden))]
+        if not spec.get("reads_other_cache", False):
+            shapes += [("k", (nkv * d, hidden)), ("v", (nkv * dv, hidden))]
+        shapes.append(("o", (hidden, nq * dv)))
+        specs = [TensorSpec(prefix + names[role], shape) for role, shape in shapes]
         if spec.get("bias", False):
-            specs += [TensorSpec(f"{prefix}{name}.bias", (shape[0],)) for name, shape in shapes]
+            specs += [TensorSpec(prefix + names[role + "_bias"], (shape[0],)) for role, shape in shapes]
+        if spec.get("sink", False):
+            specs.append(TensorSpec(prefix + names["sink"], (nq,)))
         return specs
 
     def load(self, weights, prefix):
         # The rows of the fused q/k/v weight are stored with the two elements of a rotation pair
         # side by side when the position encoding is a rotation table: the product of few rows then
         # rotates and writes the cache itself; the kernels that read its output know the order.
+        # (Not on the route for any sizes, whose kernel takes the columns in their natural order.)
         table = self.position.rotary_table()
-        self.paired = table is not None
+        self.paired = table is not None and not self.general
         order = ops.paired_rows(self.nq, self.nkv, self.d, table[1]).to(self.device) if self.paired else None
+        names = self.names
+        roles = ("q",) if self.reads_other_cache else ("q", "k", "v")
 
         def cat(suffix):
-            joined = torch.cat([weights[f"{prefix}{name}_proj.{suffix}"] for name in "qkv"], dim=0)
+            joined = torch.cat([weights[prefix + names[role + suffix]] for role in roles], dim=0)
             return joined[order].contiguous() if order is not None else joined
         keep = partial(keep_in, weights)
-        self.qkv = Linear(cat("weight"), cat("bias") if self.bias else None, self.dtype, keep=keep)
-        self.o = Linear(weights[prefix + "o_proj.weight"], weights.get(prefix + "o_proj.bias") if self.bias else None,
+        self.qkv = Linear(cat(""), cat("_bias") if self.bias else None, self.dtype, keep=keep)
+        self.o = Linear(weights[prefix + names["o"]], weights.get(prefix + names["o_bias"]) if self.bias else None,
                         self.dtype, keep=keep)
+        if self.has_sink:
+            self.sink = keep(weights[prefix + names["sink"]].float().contiguous())     # (it enters the softmax, which is float)
 
     @property
     def graph_safe(self) -> bool:
@@ -84,18 +121,45 @@ class Attention(Mixer):
             return True
         return bool(getattr(self.position, "graph_safe", False))
 
-    adds_to_residual = True
+    @property
+    def adds_to_residual(self) -> bool:
+        return not self.general
 
     def takes_normed_rows(self, rows: int) -> bool:
-        return self.qkv.takes_rows(rows)
+        return not self.general and self.qkv.takes_rows(rows)
 
     def cache_need(self):
         """A page holds two planes per kv head, [2, nkv, page_size * d]: the rotated keys as
         [position][dim] and the values transposed, [dim][position], which is how the attention
-        kernels want them as matrix operands (`ops.rope_cache` writes them so)."""
-        return CacheNeed((2, self.nkv), self.d, int(self.window) if self.window is not None else None)
+        kernels want them as matrix operands (`ops.rope_cache` writes them so).  With value heads of a
+        size dv of their own a page is [nkv, page_size * (d + dv)]: the planes of keys, then those of values."""
+        keep = self.window if self.window is not None else self.chunk       # (a chunk's first position is never further back)
+        if "cache_window" in self.spec.params:
+            keep = self.spec["cache_window"]
+        keep = int(keep) if keep is not None else None
+        if self.dv != self.d:
+            return CacheNeed((self.nkv,), self.d + self.dv, keep)
+        return CacheNeed((2, self.nkv), self.d, keep)
+
+    def _forward_general(self, x, ctx, binding: Binding):
+        """Any sizes and masks: the product, a kernel that rotates (if there is a rotation) and places q, k
+        and v, the plain attention kernel (softmax and scores float), the output product."""
+        pages = ctx.groups[binding.group]
+        table = self.position.rotary_table()
+        if table is None and type(self.position).apply_qk is not PositionEncoding.apply_qk:
+            raise invalid_config("attention: a position encoding that is no rotation table goes with the plain options only")
+        inv_freq, rot_dim = table if table is not None else (None, 0)
+        writes = binding.writes and not self.reads_other_cache
+        q = ops.qkv_place(ops.as_product(self.qkv(x)), ctx.positions, pages.slot_map if writes else ctx.no_slots, inv_freq,
+                          rot_dim, binding.cache, self.nq, 0 if self.reads_other_cache else self.nkv, self.d, self.dv, self.dtype)
+        attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq, self.nkv,
+                                         self.d, self.window, self.scale, tiled=ops.attention_generic_plan(ctx, self.d, self.dv),
+                                         seq_start=ctx.seq_start, value_dim=self.dv, chunk=self.chunk, sink=self.sink)
+        return self.o(attended)
 
     def forward(self, x, ctx, binding: Binding, into=None):
+        if self.general:
+            return self._forward_general(x, ctx, binding)
         pages = ctx.groups[binding.group]
         slot_map = pages.slot_map if binding.writes else ctx.no_slots
         table = self.position.rotary_table()

@@ -25,7 +25,8 @@ from typing import Any
 import torch
 
 from ..config.spec import PartSpec, TensorSpec
-from ..ops import NormedRows, Product, ResidualUpdated, as_product
+from .. import ops as _ops
+from ..ops import NormedDelta, NormedRows, Product, ResidualUpdated, as_product
 
 
 @dataclass(frozen=True)
@@ -108,9 +109,20 @@ class Norm(Part):
 
     def add_forward(self, residual: torch.Tensor, delta, rows: torch.Tensor | None = None, lazy: bool = False):
         """Unfused default: add in place, then norm; with `rows`, norm those rows of the sum only.
-        `delta` may be a `ResidualUpdated`: then the residual already holds it."""
+        `delta` may be a `ResidualUpdated`: then the residual already holds it; or a `NormedDelta`:
+        then its norm is applied before the add."""
         if isinstance(delta, ResidualUpdated):
             delta = None
+        if isinstance(delta, NormedDelta):
+            if rows is None:
+                _ops.norm_add_rmsnorm(residual, delta.product, delta.weight, delta.eps, None, delta.eps, self.dtype)
+                delta = None
+            else:
+                # only the wanted rows, the residual left as it was: on a copy of those rows
+                picked = residual[rows.long()].contiguous()
+                part = Product(delta.product.dense(torch.float32)[rows.long()].contiguous(), 1)
+                _ops.norm_add_rmsnorm(picked, part, delta.weight, delta.eps, None, delta.eps, self.dtype)
+                return self.forward(picked)
         if rows is not None:
             picked = residual[rows.long()]
             if delta is not None:

@@ -114,3 +114,97 @@ class PreNormBlock:
         keep("mlp_output", dense(out))
         keep("output", residual + dense(out))
         return out
+
+
+@register("block", "sandwich_norm")
+class SandwichNormBlock:
+    """x += post1(mixer(pre1(x))), then, if the layer has a feed-forward, x += post2(feed_forward(pre2(x))):
+    every sublayer's result is normed before it joins the residual.  The block does neither add itself:
+    a result waits, with its norm's weight, as a `NormedDelta`, and whoever norms the residual next
+    (this block's second norm, the next block's first, the model's last) norms it, adds it and norms
+    the sum in one kernel.  The post norms must be foldable that way (`lazy_params`)."""
+
+    _NORMS = ("mixer_norm", "mixer_post_norm", "feed_forward_norm", "feed_forward_post_norm")
+
+    def __init__(self, layer: LayerSpec, dtype, device):
+        from ..errors import invalid_config
+        self.layer = layer
+        self.dtype = dtype
+        if layer.mixer_post_norm is None:
+            raise invalid_config("a sandwich_norm layer needs a norm after its mixer")
+        if layer.feed_forward is not None and layer.feed_forward_post_norm is None:
+            raise invalid_config("a sandwich_norm layer with a feed-forward needs a norm after it")
+
+        def norm(spec):
+            return lookup("norm", spec.kind)(spec, dtype, device)
+        self.mixer_norm = norm(layer.mixer_norm)
+        self.mixer = lookup("mixer", layer.mixer.kind)(layer.mixer, dtype, device)
+        self.mixer_post_norm = norm(layer.mixer_post_norm)
+        self.feed_forward = self.feed_forward_norm = self.feed_forward_post_norm = None
+        if layer.feed_forward is not None:
+            self.feed_forward_norm = norm(layer.feed_forward_norm)
+            self.feed_forward = lookup("feed_forward", layer.feed_forward.kind)(layer.feed_forward, dtype, device)
+            self.feed_forward_post_norm = norm(layer.feed_forward_post_norm)
+        for post in (self.mixer_post_norm, self.feed_forward_post_norm):
+            if post is not None and post.lazy_params() is None:
+                raise invalid_config("a sandwich_norm layer's post norms must be RMS norms that can be folded into the add")
+
+    @classmethod
+    def _parts(cls, layer: LayerSpec):
+        """(attribute, registry table) of the parts this layer has, in the order they run."""
+        parts = [("mixer_norm", "norm"), ("mixer", "mixer"), ("mixer_post_norm", "norm")]
+        if layer.feed_forward is not None:
+            parts += [("feed_forward_norm", "norm"), ("feed_forward", "feed_forward"), ("feed_forward_post_norm", "norm")]
+        return parts
+
+    @classmethod
+    def tensor_specs(cls, layer: LayerSpec):
+        specs = []
+        for attribute, table in cls._parts(layer):
+            part_spec = getattr(layer, attribute)
+            specs += lookup(table, part_spec.kind).tensor_specs(part_spec, layer.prefix + getattr(layer, attribute + "_place"))
+        return specs
+
+    def load(self, weights):
+        for attribute, _ in self._parts(self.layer):
+            getattr(self, attribute).load(weights, self.layer.prefix + getattr(self.layer, attribute + "_place"))
+
+    def entry_norm(self):
+        """None: what is written into the residual before this block is not this block's first norm's
+        input yet (a result may still wait to be normed and added)."""
+        return None
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(getattr(self, attribute), "graph_safe", False) for attribute, _ in self._parts(self.layer))
+
+    def forward(self, residual, pending, ctx, binding, next_norm=None):
+        """A step that keeps a trace leaves, under `ctx.trace_prefix`, "input_norm", "attention_output"
+        (the mixer's result before its norm), and with a feed-forward "post_attention_norm" and
+        "mlp_output" (before its norm), then "output", the residual after the layer; it brings
+        the residual up to date itself and hands on nothing."""
+        trace = getattr(ctx, "trace", None)
+
+        def keep(name, tensor):
+            if trace is not None:
+                trace[ctx.trace_prefix + name] = tensor.float().clone()
+
+        def waiting(result, post):
+            weight, eps = post.lazy_params()
+            return ops.NormedDelta(as_product(result), weight, eps)
+        normed = self.mixer_norm.add_forward(residual, pending)
+        keep("input_norm", normed)
+        out = waiting(self.mixer.forward(normed, ctx, binding), self.mixer_post_norm)
+        if trace is not None:
+            keep("attention_output", out.product.dense(torch.float32))
+        if self.feed_forward is not None:
+            normed = self.feed_forward_norm.add_forward(residual, out)
+            keep("post_attention_norm", normed)
+            out = waiting(self.feed_forward.forward(normed, ctx), self.feed_forward_post_norm)
+            if trace is not None:
+                keep("mlp_output", out.product.dense(torch.float32))
+        if trace is None:
+            return out
+        ops.norm_add_rmsnorm(residual, out.product, out.weight, out.eps, None, out.eps, self.dtype)
+        keep("output", residual)
+        return None

@@ -1,0 +1,118 @@
+"""Latent attention: keys and values of all heads are functions of one low-rank vector per position,
+and only that vector (and one small rotated key part that all heads share) is cached.
+
+Per token, from the mixer's input h:
+    q        = W_q h, per head [plain dims | rot dims]; the rot dims are rotated by the position
+    [x | r]  = W_down h;  c = RMSNorm(x) * w (rank dims);  r (rot dims) is rotated by the position
+    per head: key = [W_uk c | r], value = W_uv c;  score = (q . key) * scale;  causal softmax with a sink
+    out      = W_o concat(heads)
+The cache keeps c and the rotated r.  Since q_plain . (W_uk c) = (W_uk^T q_plain) . c, a head's query is
+taken to the latent space before the attention (one small product per head), the attention runs over a
+single key head of rank + rot dims whose values are the c themselves, and W_uv is applied per head to the
+attended latent vector afterwards: the same sums in another order, and no key or value is ever expanded
+for a cached position.  A page holds the rows [c | r] and, for the value side, c once more, transposed.
+"""
+from __future__ import annotations
+
+import math
+from functools import partial
+
+import torch
+
+from .. import ops
+from ..config.spec import PartSpec, TensorSpec
+from ..errors import invalid_config
+from ..registry import lookup, register
+from ..weights.arena import keep_in
+from .base import Binding, CacheNeed, Mixer
+from .linear import Linear
+
+
+@register("mixer", "latent_attention")
+class LatentAttention(Mixer):
+    """spec: hidden_size, num_heads, head_dim (a head's unrotated query/key dims), rot_dim (its rotated
+    ones), value_dim, rank (of the latent vector), scale, norm_eps (of the latent vector's norm), sink (a
+    learned number per head in the softmax's denominator), position (a rotation table over rot_dim),
+    names (the tensors' names after the prefix, by role).
+    Tensors: q [H * (head_dim + rot_dim), hidden], down [rank + rot_dim, hidden], down_norm [rank],
+    up_keys [H * head_dim, rank], up_values [H * value_dim, rank], o [hidden, H * value_dim], sink [H]."""
+    graph_safe = True
+    NAMES = {"q": "q_proj.weight", "down": "kv_a_proj.weight", "down_norm": "kv_a_layernorm.weight",
+             "up_keys": "k_b_proj.weight", "up_values": "v_b_proj.weight", "o": "o_proj.weight", "sink": "sinks"}
+
+    def __init__(self, spec: PartSpec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.hidden = int(spec["hidden_size"])
+        self.heads = int(spec["num_heads"])
+        self.plain = int(spec["head_dim"])
+        self.rot = int(spec["rot_dim"])
+        self.dv = int(spec["value_dim"])
+        self.rank = int(spec["rank"])
+        self.scale = float(spec.get("scale") or 1.0 / math.sqrt(float(self.plain + self.rot)))
+        self.norm_eps = float(spec["norm_eps"])
+        self.has_sink = bool(spec.get("sink", False))
+        if min(self.heads, self.plain, self.dv, self.rank) <= 0 or self.rot < 0 or self.rot % 2 != 0:
+            raise invalid_config("latent_attention: sizes must be positive, rot_dim even")
+        if self.rank > ops.ATTENTION_MAX_HEAD_DIM:
+            raise invalid_config(f"latent_attention: a latent vector of {self.rank} dims is beyond the attention kernel's "
+                                 f"{ops.ATTENTION_MAX_HEAD_DIM} value dims")
+        self.inv_freq = None
+        if self.rot > 0:
+            position = spec["position"]
+            table = lookup("position_encoding", position.kind)(position, dtype, device).rotary_table()
+            if table is None or table[1] != self.rot:
+                raise invalid_config("latent_attention: the position encoding must be a rotation table over rot_dim")
+            self.inv_freq = table[0]
+        self.names = {**self.NAMES, **dict(spec.get("names") or {})}
+        self.first = self.o = self.down_norm = self.up_keys = self.up_values_t = self.sink = None
+
+    @classmethod
+    def tensor_specs(cls, spec, prefix):
+        names = {**cls.NAMES, **dict(spec.get("names") or {})}
+        hidden, heads, plain, rot = int(spec["hidden_size"]), int(spec["num_heads"]), int(spec["head_dim"]), int(spec["rot_dim"])
+        dv, rank = int(spec["value_dim"]), int(spec["rank"])
+        specs = [TensorSpec(prefix + names["q"], (heads * (plain + rot), hidden)),
+                 TensorSpec(prefix + names["down"], (rank + rot, hidden)),
+                 TensorSpec(prefix + names["down_norm"], (rank,), init="norm"),
+                 TensorSpec(prefix + names["up_keys"], (heads * plain, rank)),
+                 TensorSpec(prefix + names["up_values"], (heads * dv, rank)),
+                 TensorSpec(prefix + names["o"], (hidden, heads * dv))]
+        if spec.get("sink", False):
+            specs.append(TensorSpec(prefix + names["sink"], (heads,)))
+        return specs
+
+    def load(self, weights, prefix):
+        names, keep = self.names, partial(keep_in, weights)
+        # one product for the queries and the down projection
+        self.first = Linear(torch.cat([weights[prefix + names["q"]], weights[prefix + names["down"]]], dim=0), None, self.dtype, keep=keep)
+        self.down_norm = keep(weights[prefix + names["down_norm"]].contiguous())
+        # per head, as the block-diagonal product wants them, [inner, outer]: a head's query goes to the latent
+        # space through W_uk^T (W_uk is [plain, rank] per head: already [inner, outer]); its attended latent
+        # vector to its values through W_uv ([value_dim, rank] per head: transposed here)
+        self.up_keys = keep(weights[prefix + names["up_keys"]].reshape(self.heads, self.plain, self.rank).contiguous())
+        self.up_values_t = keep(weights[prefix + names["up_values"]].reshape(self.heads, self.dv, self.rank).transpose(1, 2).contiguous())
+        self.o = Linear(weights[prefix + names["o"]], None, self.dtype, keep=keep)
+        if self.has_sink:
+            self.sink = keep(weights[prefix + names["sink"]].float().contiguous())
+
+    def cache_need(self):
+        """One key head of rank + rot dims, [row][dim], then its rank value dims transposed, [dim][row]."""
+        return CacheNeed((1,), 2 * self.rank + self.rot, None)
+
+    def forward(self, x, ctx, binding: Binding, into=None):
+        pages = ctx.groups[binding.group]
+        key = self.rank + self.rot
+        fused = ops.as_product(self.first(x))
+        tokens = fused.rows
+        q_plain, q_wide = ops.latent_place(fused, ctx.positions, pages.slot_map if binding.writes else ctx.no_slots, self.inv_freq,
+                                           self.down_norm, self.norm_eps, binding.cache, self.heads, self.plain, self.rot,
+                                           self.rank, self.dtype)
+        ops.block_linear(q_plain, 0, self.heads * self.plain, self.plain, self.up_keys, None,
+                         q_wide, 0, self.heads * key, key, tokens)
+        attended = ops.attention_generic(q_wide, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.heads, 1,
+                                         key, None, self.scale, tiled=ops.attention_generic_plan(ctx, key, self.rank),
+                                         seq_start=ctx.seq_start, value_dim=self.rank, sink=self.sink)
+        values = torch.empty((tokens, self.heads * self.dv), dtype=self.dtype, device=attended.device)
+        ops.block_linear(attended, 0, self.heads * self.rank, self.rank, self.up_values_t, None,
+                         values, 0, self.heads * self.dv, self.dv, tokens)
+        return self.o(values)

@@ -19,38 +19,60 @@ from .linear import Linear
 
 @register("feed_forward", "gated_mlp")
 class GatedMLP(FeedForward):
-    """spec: hidden_size, intermediate_size, activation ("silu").
-    Tensors: `<prefix>{gate,up,down}_proj.weight`."""
+    """spec: hidden_size, intermediate_size, activation: "silu" (silu(gate) * up), or "clamped_swish" with
+    `alpha` and `limit`: g = min(gate, limit), u = clamp(up, -limit, limit), g * sigmoid(alpha * g) * (u + 1);
+    optionally bias (all three products have one) and names (the tensors' names after the prefix, by role:
+    gate, up, down, gate_bias, up_bias, down_bias).
+    Tensors: `<prefix>{gate,up,down}_proj.weight` unless `names` says otherwise."""
     graph_safe = True
+    NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight",
+             "gate_bias": "gate_proj.bias", "up_bias": "up_proj.bias", "down_bias": "down_proj.bias"}
 
     def __init__(self, spec: PartSpec, dtype, device):
         super().__init__(spec, dtype, device)
         self.hidden = int(spec["hidden_size"])
         self.inter = int(spec["intermediate_size"])
-        if spec.get("activation", "silu") != "silu":
-            raise invalid_config(f"gated_mlp: activation '{spec['activation']}' is not implemented")
+        self.activation = spec.get("activation", "silu")
+        if self.activation not in ops.GATES:
+            raise invalid_config(f"gated_mlp: activation '{self.activation}' is not implemented")
+        self.alpha, self.limit = float(spec.get("alpha", 1.0)), float(spec.get("limit", 0.0))
+        if self.activation == "clamped_swish" and not self.limit > 0.0:
+            raise invalid_config("gated_mlp: the clamped gate needs a positive limit")
+        self.bias = bool(spec.get("bias", False))
+        self.names = {**self.NAMES, **dict(spec.get("names") or {})}
         self.gate_up = self.down = None
 
     @classmethod
     def tensor_specs(cls, spec, prefix):
+        names = {**cls.NAMES, **dict(spec.get("names") or {})}
         hidden, inter = int(spec["hidden_size"]), int(spec["intermediate_size"])
-        return [TensorSpec(prefix + "gate_proj.weight", (inter, hidden)),
-                TensorSpec(prefix + "up_proj.weight", (inter, hidden)),
-                TensorSpec(prefix + "down_proj.weight", (hidden, inter))]
+        shapes = (("gate", (inter, hidden)), ("up", (inter, hidden)), ("down", (hidden, inter)))
+        specs = [TensorSpec(prefix + names[role], shape) for role, shape in shapes]
+        if spec.get("bias", False):
+            specs += [TensorSpec(prefix + names[role + "_bias"], (shape[0],)) for role, shape in shapes]
+        return specs
 
     def load(self, weights, prefix):
-        gate, up = weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]
+        names = self.names
+        gate, up = weights[prefix + names["gate"]], weights[prefix + names["up"]]
         keep = partial(keep_in, weights)
-        self.gate_up = Linear(torch.stack([gate, up], dim=1).reshape(2 * self.inter, self.hidden), None, self.dtype, keep=keep)
-        self.down = Linear(weights[prefix + "down_proj.weight"], None, self.dtype, keep=keep)
+        bias = down_bias = None
+        if self.bias:
+            bias = torch.stack([weights[prefix + names["gate_bias"]], weights[prefix + names["up_bias"]]], dim=1).reshape(2 * self.inter)
+            down_bias = weights[prefix + names["down_bias"]]
+        self.gate_up = Linear(torch.stack([gate, up], dim=1).reshape(2 * self.inter, self.hidden), bias, self.dtype, keep=keep)
+        self.down = Linear(weights[prefix + names["down"]], down_bias, self.dtype, keep=keep)
 
-    adds_to_residual = True
+    @property
+    def adds_to_residual(self) -> bool:
+        return True
 
     def takes_normed_rows(self, rows: int) -> bool:
-        return self.gate_up.takes_rows(rows)
+        return self.activation == "silu" and self.gate_up.takes_rows(rows)
 
     def forward(self, x, ctx, into=None):
-        hidden = self.gate_up(x, gated=True)
+        # (the products that apply the gate themselves know the SiLU gate only)
+        hidden = self.gate_up(x, gated=self.activation == "silu")
         if isinstance(hidden, ops.Product):
-            hidden = ops.silu_mul(hidden, self.dtype, interleaved=True)
+            hidden = ops.silu_mul(hidden, self.dtype, interleaved=True, gate=self.activation, alpha=self.alpha, limit=self.limit)
         return self.down(hidden, into=into)

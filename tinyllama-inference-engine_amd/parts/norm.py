@@ -9,26 +9,34 @@ from .. import ops
 from ..config.spec import PartSpec, TensorSpec
 from ..registry import register
 from ..weights.arena import keep_in
-from .base import Norm, ResidualUpdated, as_product
+from .base import Norm, NormedDelta, ResidualUpdated, as_product
 
 
 @register("norm", "rms_norm")
 class RMSNorm(Norm):
-    """spec: size, eps.  Tensor: `<prefix>weight` [size]."""
+    """spec: size, eps; optionally offset (the stored weight w lies around zero and acts as 1 + w) and
+    tensor (the tensor's name after the prefix; default "weight").  Tensor: `<prefix><tensor>` [size]."""
     graph_safe = True
 
     def __init__(self, spec: PartSpec, dtype, device):
         super().__init__(spec, dtype, device)
         self.size = int(spec["size"])
         self.eps = float(spec["eps"])
+        self.offset = bool(spec.get("offset", False))
         self.weight = None
 
     @classmethod
     def tensor_specs(cls, spec, prefix):
-        return [TensorSpec(prefix + "weight", (int(spec["size"]),), init="norm")]
+        name = prefix + str(spec.get("tensor", "weight"))
+        return [TensorSpec(name, (int(spec["size"]),), init="offset" if spec.get("offset", False) else "norm")]
 
     def load(self, weights, prefix):
-        self.weight = keep_in(weights, weights[prefix + "weight"].contiguous())
+        stored = weights[prefix + str(self.spec.get("tensor", "weight"))]
+        if self.offset:
+            # 1 + w is formed once, in float, and kept so: bfloat16 would round the sum (near 1) to 8 bits
+            self.weight = keep_in(weights, (1.0 + stored.float()).contiguous())
+        else:
+            self.weight = keep_in(weights, stored.contiguous())
 
     def forward(self, residual):
         return ops.add_rmsnorm(residual, None, self.weight, self.eps, self.dtype)
@@ -43,5 +51,10 @@ class RMSNorm(Norm):
             if lazy and rows is None and delta.normed is not None:
                 return delta.normed
             delta = None
+        if isinstance(delta, NormedDelta):
+            if delta.weight.dtype == self.weight.dtype:
+                return ops.norm_add_rmsnorm(residual, delta.product, delta.weight, delta.eps, self.weight, self.eps,
+                                            self.dtype, rows=rows)
+            return super().add_forward(residual, delta, rows=rows)      # weights of two types: the add, then this norm
         product = as_product(delta) if delta is not None else None
         return ops.add_rmsnorm(residual, product, self.weight, self.eps, self.dtype, rows=rows)

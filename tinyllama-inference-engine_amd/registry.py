@@ -43,13 +43,16 @@ def lookup(table: str, name: str):
 
 
 def config_from_dict(raw: Mapping[str, Any]):
-    """Chooses the configuration class by `architectures[0]`; without that key, by
-    `model_type` == "llama" (the only key the reference checks, src/model_config.cpp:25-27)."""
+    """Chooses the configuration class by `architectures[0]`, or by `architecture` (one name, as some
+    configurations write it); without those keys, by `model_type` == "llama" (the only key the
+    reference checks, src/model_config.cpp:25-27)."""
     architectures = raw.get("architectures")
     if isinstance(architectures, list) and architectures and isinstance(architectures[0], str):
         name = architectures[0]
+    elif isinstance(raw.get("architecture"), str):
+        name = raw["architecture"]
     elif raw.get("model_type") == "llama":
         name = "LlamaForCausalLM"
     else:
-        raise invalid_config("config.json names no architecture ('architectures' or model_type 'llama')")
+        raise invalid_config("config.json names no architecture ('architectures', 'architecture' or model_type 'llama')")
     return lookup("architecture", name).from_dict(raw)

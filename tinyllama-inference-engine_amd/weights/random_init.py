@@ -39,6 +39,8 @@ def _draw(spec: TensorSpec, seed: int, std: float, norm_std: float, dtype: torch
         values = values * std
     elif spec.init == "norm":
         values = 1.0 + values * norm_std
+    elif spec.init == "offset":
+        values = values * norm_std
     elif spec.init == "zeros":
         values = torch.zeros(spec.shape, device=device)
     else:
