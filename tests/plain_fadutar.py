@@ -150,7 +150,7 @@ def plain_causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: torch.Tensor) -
     tokens, n = x.shape[0], taps.shape[1]
     x, taps = x.double(), taps.double()
     out = bias.double().expand(tokens, -1).clone()
-    for j in range(n):
+    for j in range(min(n, tokens)):                 # (a tap further back than the sequence is long meets zeros only)
         out[j:] += taps[:, n - 1 - j] * x[:tokens - j]
     return out
 
