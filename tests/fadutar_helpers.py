@@ -31,6 +31,10 @@ CONFIG_P = {
         {"type": "latent_attention", "mixer": {"heads": 3, "dim": 24, "rot_dim": 8, "vdim": 16, "kv_rank": 40, "scale": 0.17,
                                                "rot": {"base": 10000.0, "dims": 8}}, "mlp": _mlp(160, 0.75)},
         {"type": "attention", "mixer": {"heads": 2, "kv_heads": 2, "dim": 72, "vdim": 8, "scale": 0.1}, "mlp": None},
+        # one head size for keys and values, a multiple of 16: in bfloat16 these two take the kernel on the matrix cores
+        {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 0.2, "mask": {"size": 48}},
+         "mlp": _mlp(64, 2.0)},
+        {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 0.15, "kv_from": 5}, "mlp": None},
     ],
 }
 CONFIG_Q = {

@@ -20,11 +20,14 @@ from tlie_amd.weights.store import WeightStore
 def test_the_architecture_is_found_by_its_name_and_turned_into_data():
     spec = config_from_dict(CONFIG_P).to_spec()
     assert spec.architecture == "Fadutar" and spec.max_positions is None
-    assert [layer.block for layer in spec.layers] == ["sandwich_norm"] * 5
-    assert [layer.mixer.kind for layer in spec.layers] == ["gated_recurrence", "attention", "attention", "latent_attention", "attention"]
-    assert [layer.feed_forward is None for layer in spec.layers] == [True, False, False, False, True]
+    assert [layer.block for layer in spec.layers] == ["sandwich_norm"] * 7
+    assert [layer.mixer.kind for layer in spec.layers] == ["gated_recurrence", "attention", "attention", "latent_attention",
+                                                          "attention", "attention", "attention"]
+    assert [layer.feed_forward is None for layer in spec.layers] == [True, False, False, False, True, False, True]
     # the layer that reads another layer's keys and values runs on that layer's cache and owns none
-    assert [(run.layer, run.cache_of) for run in spec.runs] == [(0, 0), (1, 1), (2, 1), (3, 3), (4, 4)]
+    assert [(run.layer, run.cache_of) for run in spec.runs] == [(0, 0), (1, 1), (2, 1), (3, 3), (4, 4), (5, 5), (6, 5)]
+    # a cache whose reader sees every earlier position keeps its pages for good, whatever its owner's chunks
+    assert spec.layers[5].mixer["chunk"] == 48 and spec.layers[5].mixer["cache_window"] is None
     owner, reader, free = spec.layers[1].mixer, spec.layers[2].mixer, spec.layers[4].mixer
     assert owner["chunk"] == 24 and reader["chunk"] == 40 and free["chunk"] is None
     assert owner["cache_window"] == 40          # kept for as long as the reader's wider chunks reach

@@ -153,6 +153,54 @@ def test_attention_with_sink_and_chunks(heads, groups, d, dv, chunk, page_size):
         assert float((got.cpu().double() - want).abs().max()) < 2e-5, f"cut {cuts}"
 
 
+def _attend_matrix_cores(q, k, v, sink, scale, chunk, page_size, cuts):
+    """The same through the kernel on the matrix cores (bfloat16, one head size), launched as the part
+    launches it: a work list for steps of several tokens, none for single tokens, keys cut into parts
+    as the kernel's own policy says."""
+    from types import SimpleNamespace
+    import numpy as np
+    from tlie_amd import ops
+    tokens, heads, d = q.shape
+    groups = k.shape[1]
+    blocks = (tokens + page_size - 1) // page_size
+    order = list(range(blocks + 3))
+    random.Random(blocks).shuffle(order)
+    cache = torch.zeros((blocks + 3, 2, groups, page_size * d), dtype=torch.bfloat16, device=DEVICE)
+    table = torch.tensor([order[:blocks]], dtype=torch.int32, device=DEVICE)
+    outs, at, index = [], 0, 0
+    while at < tokens:
+        count = min(cuts[index % len(cuts)], tokens - at)
+        index += 1
+        positions = torch.arange(at, at + count, dtype=torch.int32, device=DEVICE)
+        slots = torch.tensor([order[p // page_size] * page_size + p % page_size for p in range(at, at + count)], dtype=torch.int32, device=DEVICE)
+        fused = torch.cat([q[at:at + count].reshape(count, -1), k[at:at + count].reshape(count, -1), v[at:at + count].reshape(count, -1)], dim=1)
+        placed = ops.qkv_place(ops.Product(fused.to(DEVICE).contiguous(), 1), positions, slots, None, 0, cache, heads, groups, d, d, torch.bfloat16)
+        host = {"seq_start": np.asarray([0, count], dtype=np.int32), "seq_len": np.asarray([at + count], dtype=np.int32)}
+        ctx = SimpleNamespace(max_new=count, num_seqs=1, num_tokens=count, max_context=at + count, scratch={}, tile_owner=None,
+                              compute_units=256, host=host, tokens=positions)
+        tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, heads // groups, groups, d)
+        outs.append(ops.attention_mfma(placed, cache, table, tiles, positions, heads, groups, d, None, scale, nsplit, split_len, col_tiles,
+                                       waves, shared, chunk=chunk, sink=sink.to(DEVICE) if sink is not None else None))
+        at += count
+    return torch.cat(outs, dim=0).reshape(tokens, heads, d)
+
+
+@pytest.mark.parametrize("heads,groups,d,chunk,page_size,tokens", [(4, 2, 32, 48, 16, 300), (8, 1, 64, 100, 16, 1000), (2, 2, 16, 33, 32, 200),
+                                                                   (6, 3, 128, None, 16, 300), (4, 4, 48, 64, 16, 900)])
+def test_attention_on_the_matrix_cores_with_sink_and_chunks(heads, groups, d, chunk, page_size, tokens):
+    generator = torch.Generator().manual_seed(d + tokens)
+    q, k, v = (torch.randn(tokens, n, d, generator=generator).bfloat16().float() for n in (heads, groups, groups))
+    sink = torch.randn(heads, generator=generator) + 1.0
+    want = plain_sink_attention(q, k, v, sink, 0.2, chunk)
+    for cuts in ([tokens], [1], [tokens - 40] + [1] * 40, [37, 2, 5, 1, 130]):
+        if cuts == [1] and tokens > 300:
+            continue
+        got = _attend_matrix_cores(q, k, v, sink, 0.2, chunk, page_size, cuts)
+        assert float((got.float().cpu().double() - want).abs().max()) < 3e-2, f"cut {cuts[:5]}"
+    # the sink taken away changes the result by far more than that: it is not a detail within the tolerance
+    assert float((plain_sink_attention(q, k, v, sink - 30.0, 0.2, chunk) - want).abs().max()) > 0.2
+
+
 def test_a_sink_that_is_left_out_and_a_key_past_the_chunk_edge_show():
     """Weights made so that faults show: one query and one key are scaled so that their score towers over
     all others; just inside the query's chunk that key takes nearly all the weight, just outside it none;

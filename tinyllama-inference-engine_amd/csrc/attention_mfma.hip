@@ -102,8 +102,16 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
                       const int* __restrict__ block_table, int max_blocks, const int4* __restrict__ tiles,
                       const int* __restrict__ positions, uint16_t* __restrict__ out, float* __restrict__ part_o,
                       float* __restrict__ part_ml, int nsplit, int split_len, int nq, int nkv, int page_size,
-                      int window, float scale_log2, int round_size) {
+                      int window, int chunk, const float* __restrict__ sink, float scale_log2, int round_size) {
   constexpr int D = DT * 16;
+  // the first key that the token at position p sees: the window's edge, or the start of the token's own
+  // chunk of positions (chunks are counted from position 0), whichever is later; 0 without either
+  const bool bounded = window > 0 || chunk > 0;
+  auto lower = [&](int p) {
+    int lo = window > 0 ? max(0, p - window + 1) : 0;
+    if (chunk > 0) lo = max(lo, p - p % chunk);
+    return lo;
+  };
   constexpr int KS = (DT + 1) / 2;                 // 32-wide k steps of the first product
   const int lane = threadIdx.x & 63, col = lane & 15, grp = lane >> 4;
   const int wave = threadIdx.x >> 6, waves = blockDim.x >> 6;     // waves that share the tile's keys
@@ -152,13 +160,13 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
     tok[ct] = tok0 + (valid_col[ct] ? c / G : 0);
     head[ct] = kvh * G + (valid_col[ct] ? c % G : 0);
     pos_col[ct] = valid_col[ct] ? pos0 + c / G : -1;
-    lo_col[ct] = window > 0 ? max(0, pos_col[ct] - window + 1) : 0;
+    lo_col[ct] = bounded ? lower(pos_col[ct]) : 0;
   }
 
   // the tile's key range, and this split's part of it
   const int last_col = min(col0 + 16 * CT - 1, ncols - 1);
   const int tile_hi = pos0 + last_col / G + 1;
-  const int tile_lo = window > 0 ? max(0, pos0 + col0 / G - window + 1) : 0;
+  const int tile_lo = bounded ? lower(pos0 + col0 / G) : 0;
   const int split_lo = nsplit > 1 ? split * split_len : 0;
   const int range_lo = __builtin_amdgcn_readfirstlane(wave_active ? max(tile_lo, split_lo) : 0);
   const int range_hi = __builtin_amdgcn_readfirstlane(wave_active ? (nsplit > 1 ? min(tile_hi, split_lo + split_len) : tile_hi) : 0);
@@ -350,11 +358,11 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   // split_lo & ~31 whatever the position), so some may lie past the range: they are safe (see
   // above) and unused.
   constexpr int NB = (CT == 1 && DT <= 4) ? 4 : 2;
-  const int first_block = ((window > 0 ? range_lo : split_lo) & ~31) + 32 * wave;
+  const int first_block = ((bounded ? range_lo : split_lo) & ~31) + 32 * wave;
   const int stride = 32 * waves;
   // a block that every column of the tile sees whole: inside the range, below the first column's
   // position, inside the last column's window
-  const int open_lo = __builtin_amdgcn_readfirstlane(max((range_lo + 31) & ~31, window > 0 ? tile_hi - window : 0));
+  const int open_lo = __builtin_amdgcn_readfirstlane(max((range_lo + 31) & ~31, bounded ? lower(tile_hi - 1) : 0));
   const int open_hi = __builtin_amdgcn_readfirstlane(min(range_hi, pos0 + col0 / G + 1) & ~31);
   auto work = [&](int kb, KeyBlock& block) {
     if (kb >= open_lo && kb + 32 <= open_hi)
@@ -375,7 +383,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
     constexpr int kStage = (kPieces + 255) / 256;        // pieces a thread brings (a workgroup has 256 or 512 threads)
     const int group_last = min(group_col0 + 16 * CT * waves - 1, ncols - 1);
     const int group_hi = pos0 + group_last / G + 1;
-    const int group_lo = window > 0 ? max(0, pos0 + group_col0 / G - window + 1) : 0;
+    const int group_lo = bounded ? lower(pos0 + group_col0 / G) : 0;
     const int all_lo = max(group_lo, split_lo);
     const int all_hi = nsplit > 1 ? min(group_hi, split_lo + split_len) : group_hi;
     // Blocks are asked for kAhead blocks before their turn and wait in registers: a workgroup walks
@@ -554,7 +562,14 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   for (int ct = 0; ct < CT; ++ct) {
     if (!valid_col[ct]) continue;
     if (nsplit == 1) {
-      const float inv = 1.f / running_sum[ct];
+      float inv = 1.f / running_sum[ct];
+      if (sink != nullptr) {
+        // the sink joins the denominator once, as exp(sink): in base 2 and on the common scale of the sums
+        const float own = sink[head[ct]] * 1.4426950408889634f;
+        const float top = fmaxf(running_max[ct], own);
+        const float mine = __builtin_amdgcn_exp2f(running_max[ct] - top);
+        inv = mine / (running_sum[ct] * mine + __builtin_amdgcn_exp2f(own - top));
+      }
       uint16_t* o_row = out + (static_cast<size_t>(tok[ct]) * nq + head[ct]) * D;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
@@ -584,7 +599,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
 // the weights are formed once, by the lanes, and kept in LDS.
 __global__ void __launch_bounds__(64)
 attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                       uint16_t* __restrict__ out, int nsplit, int d) {
+                       uint16_t* __restrict__ out, int nsplit, int d, const float* __restrict__ sink, int nq) {
   extern __shared__ float weight[];                  // nsplit
   const size_t row = blockIdx.x;                     // token * nq + head
   const float* ml = part_ml + row * nsplit * 2;
@@ -603,6 +618,9 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
   float top = -INFINITY;
   for (int p = lane; p < nsplit; p += 64) top = fmaxf(top, ml[p * 2]);
   top = wave_max(top);
+  // a sink (one number per head) joins the denominator once, as exp(sink), in base 2 like the maxima
+  const float own = sink != nullptr ? sink[row % nq] * 1.4426950408889634f : -INFINITY;
+  top = fmaxf(top, own);
   float total = 0.f;
   for (int p = lane; p < nsplit; p += 64) {
     const float m = ml[p * 2];
@@ -611,6 +629,7 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
     total += w * ml[p * 2 + 1];
   }
   total = wave_sum(total);
+  if (sink != nullptr) total += exp2f(own - top);
   __syncthreads();
   const float inv = 1.f / total;
   if (ahead) {
@@ -656,15 +675,15 @@ static int compute_units() {
 template <int DT, int CT, bool SHARED = false>
 static int launch_attention(const void* q, const void* cache, const int* block_table, int max_blocks, const void* tiles,
                             int num_tiles, const int* positions, void* out, float* part_o, float* part_ml, int nsplit,
-                            int split_len, int nq, int nkv, int page_size, int window, float scale, int waves,
-                            hipStream_t stream) {
+                            int split_len, int nq, int nkv, int page_size, int window, int chunk, const float* sink, float scale,
+                            int waves, hipStream_t stream) {
   const float scale_log2 = scale * 1.4426950408889634f;
   // LDS for merging the waves: their maxima and sums, and half as many slots as waves for the results
   const size_t lds = !SHARED && waves > 1 ? (static_cast<size_t>(waves) * CT * 32 + static_cast<size_t>(waves / 2) * CT * DT * 256) * sizeof(float) : 0;
   if (lds > 64 * 1024) return kBadArgument;
   hipLaunchKernelGGL((attention_mfma_kernel<DT, CT, SHARED>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
                      (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
-                     part_ml, nsplit, split_len, nq, nkv, page_size, window, scale_log2, compute_units());
+                     part_ml, nsplit, split_len, nq, nkv, page_size, window, chunk, sink, scale_log2, compute_units());
   return launch_status();
 }
 
@@ -685,7 +704,9 @@ using namespace tlie;
 static int attention_entry(const void* q, const void* cache, const int* block_table, int max_blocks,
                            const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
                            float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
-                           int d, int page_size, int window, float scale, int waves, int shared, void* stream) {
+                           int d, int page_size, int window, int chunk, const float* sink, float scale, int waves, int shared,
+                           void* stream) {
+  if (chunk < 0) return kBadArgument;
   if (num_tiles <= 0 || tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 256 || d % 16 != 0 ||
       page_size < 16 || (page_size & (page_size - 1)) != 0 || max_blocks <= 0 || nsplit < 1 || nsplit > 65535 || nkv > 65535)
     return kBadArgument;
@@ -702,7 +723,7 @@ static int attention_entry(const void* q, const void* cache, const int* block_ta
   hipStream_t s = (hipStream_t)stream;
   int status = kBadArgument;
 #define TLIE_ARGS q, cache, block_table, max_blocks, tiles, num_tiles, positions, out, part_o, part_ml, nsplit, split_len, nq, \
-                  nkv, page_size, window, scale, waves, s
+                  nkv, page_size, window, chunk, sink, scale, waves, s
 #define TLIE_CASE(DT)                                        \
   case DT:                                                   \
     status = launch_attention<DT, 1>(TLIE_ARGS);             \
@@ -743,16 +764,19 @@ static int attention_entry(const void* q, const void* cache, const int* block_ta
 #undef TLIE_ARGS
   if (status != kOk || nsplit == 1) return status;
   hipLaunchKernelGGL(attention_merge_kernel, dim3(tokens * nq), dim3(64), nsplit * sizeof(float), s, part_o, part_ml,
-                     (uint16_t*)out, nsplit, d);
+                     (uint16_t*)out, nsplit, d, sink, nq);
   return launch_status();
 }
 
 extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* block_table, int max_blocks,
                                    const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
                                    float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
-                                   int d, int page_size, int window, float scale, int waves, int shared, void* stream) {
+                                   int d, int page_size, int window, int chunk, const float* sink, float scale, int waves,
+                                   int shared, void* stream) {
+  // chunk > 0: a token sees only the keys of its own chunk of so many positions (counted from position 0);
+  // sink (or null): float [nq], a number per head whose exponential joins the softmax's denominator
   return attention_entry(q, cache, block_table, max_blocks, tiles, num_tiles, col_tiles, positions, out, part_o, part_ml, nsplit,
-                         split_len, tokens, nq, nkv, d, page_size, window, scale, waves, shared, stream);
+                         split_len, tokens, nq, nkv, d, page_size, window, chunk, sink, scale, waves, shared, stream);
 }
 
 // ---- the same attention for callers that cannot allocate (declared and described in no_alloc.h) ----------
@@ -796,5 +820,5 @@ extern "C" int tlie_attention_mfma_no_alloc(const void* q, const void* cache, co
     part_ml = reinterpret_cast<float*>(base + o_bytes);
   }
   return attention_entry(q, cache, block_table, max_blocks, tiles, num_tiles, col_tiles, positions, out, part_o, part_ml, nsplit,
-                         split_len, tokens, nq, nkv, d, page_size, window, scale, waves, shared, stream);
+                         split_len, tokens, nq, nkv, d, page_size, window, 0, nullptr, scale, waves, shared, stream);
 }

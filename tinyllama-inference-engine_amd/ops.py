@@ -946,7 +946,7 @@ def attention_mfma_takes(dtype: torch.dtype, head_dim: int, page_size: int) -> b
 def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor | None,
                    positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
                    scale: float, nsplit: int = 1, split_len: int = 0, col_tiles: int = 1, waves: int = 1,
-                   shared: bool = False) -> torch.Tensor:
+                   shared: bool = False, chunk: int | None = None, sink: torch.Tensor | None = None) -> torch.Tensor:
     """Causal attention of every token of the step over its sequence's cache, bfloat16.
 
     tiles: int32 [n, 4] from `attention_tiles` (built from the same step as block_table and
@@ -958,8 +958,16 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     workgroup share each tile's (or part's) keys and merge their results before writing.
     shared (prompt portions; col_tiles 1 or 2, head size up to 128, 4 or 8 waves): the tiles were made
     with col_tiles * waves column groups, every wave takes col_tiles of them, and each block of keys
-    and values is brought once for the whole workgroup."""
+    and values is brought once for the whole workgroup.
+    chunk: a token sees only the keys of its own chunk of so many positions (counted from position 0).
+    sink: float32 [nq], a number per head whose exponential joins the softmax's denominator."""
     _device_tensor(q, "q", torch.bfloat16)
+    if sink is not None:
+        _device_tensor(sink, "sink", torch.float32)
+        if sink.shape != (num_heads,):
+            raise invalid_shape("attention: the sink needs one entry per query head")
+    if chunk is not None and int(chunk) <= 0:
+        raise invalid_argument("attention: a chunk must be a positive count of positions")
     _device_tensor(cache, "cache", torch.bfloat16)
     _device_tensor(block_table, "block_table", torch.int32)
     _device_tensor(positions, "positions", torch.int32)
@@ -1002,7 +1010,8 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     _check(library().tlie_attention_mfma(_ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(tiles),
                                          num_tiles, col_tiles, _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), nsplit,
                                          split_len, tokens, num_heads, num_kv_heads, head_dim, page_size,
-                                         int(window) if window else 0, ctypes.c_float(scale), waves, int(bool(shared)), _stream()),
+                                         int(window) if window else 0, int(chunk) if chunk else 0, _ptr(sink),
+                                         ctypes.c_float(scale), waves, int(bool(shared)), _stream()),
            "attention_mfma")
     return out
 

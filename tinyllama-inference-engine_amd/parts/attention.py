@@ -152,9 +152,16 @@ class Attention(Mixer):
         writes = binding.writes and not self.reads_other_cache
         q = ops.qkv_place(ops.as_product(self.qkv(x)), ctx.positions, pages.slot_map if writes else ctx.no_slots, inv_freq,
                           rot_dim, binding.cache, self.nq, 0 if self.reads_other_cache else self.nkv, self.d, self.dv, self.dtype)
-        attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq, self.nkv,
-                                         self.d, self.window, self.scale, tiled=ops.attention_generic_plan(ctx, self.d, self.dv),
-                                         seq_start=ctx.seq_start, value_dim=self.dv, chunk=self.chunk, sink=self.sink)
+        if self.dv == self.d and ops.attention_mfma_takes(self.dtype, self.d, binding.cache.shape[3] // self.d):
+            # bfloat16, one head size: the kernel on the matrix cores (scores, softmax and sink float)
+            tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, self.nq // self.nkv, self.nkv, self.d)
+            attended = ops.attention_mfma(q, binding.cache, pages.block_table, tiles, ctx.positions, self.nq, self.nkv, self.d,
+                                          self.window, self.scale, nsplit, split_len, col_tiles, waves, shared,
+                                          chunk=self.chunk, sink=self.sink)
+        else:
+            attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq, self.nkv,
+                                             self.d, self.window, self.scale, tiled=ops.attention_generic_plan(ctx, self.d, self.dv),
+                                             seq_start=ctx.seq_start, value_dim=self.dv, chunk=self.chunk, sink=self.sink)
         return self.o(attended)
 
     def forward(self, x, ctx, binding: Binding, into=None):
