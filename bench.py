@@ -161,6 +161,74 @@ def run_workload(engine, torch, workload, vocab, budget, chunk, slice_steps=8, p
             "ms_step_decode_only": middle(decode_only)}
 
 
+# layer sizes for `--design fadutar`: TinyLlama's and Llama-3-8B's widths, heads and feed-forwards; the latent layers'
+# rank and rotated part after the ratios of published latent-attention models, within the 256 value dims the
+# plain attention kernel takes; the recurrence as wide as the model
+DESIGN_SIZES = {
+    "w2048": dict(width=2048, ff=5632, heads=32, kv_heads=4, dim=64, chunk=1024, latent_heads=32, latent_dim=64, latent_rot=32,
+                  latent_vdim=64, rank=128, lru_width=2048, lru_blocks=8, taps=4, vocab=32000, groups=2),
+    "w4096": dict(width=4096, ff=14336, heads=32, kv_heads=8, dim=128, chunk=1024, latent_heads=32, latent_dim=128, latent_rot=64,
+                  latent_vdim=128, rank=192, lru_width=4096, lru_blocks=16, taps=4, vocab=32000, groups=1),
+}
+
+
+def design_configs(sizes):
+    """(the Fadutar configuration, the Llama configuration of equal sizes): `groups` times the four kinds of layer
+    (chunked attention, attention on that layer's keys and values, latent attention, recurrence), each with a
+    feed-forward, beside as many Llama layers of the same width, heads and feed-forward."""
+    s = sizes
+    mlp = {"kind": "dense", "ff": s["ff"], "limit": 7.0}
+    attention = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5,
+                 "mask": {"size": s["chunk"]}}
+    layers = []
+    for group in range(s["groups"]):
+        layers += [
+            {"type": "attention", "mixer": dict(attention), "mlp": mlp},
+            {"type": "attention", "mixer": dict(attention, kv_from=4 * group), "mlp": mlp},
+            {"type": "latent_attention", "mixer": {"heads": s["latent_heads"], "dim": s["latent_dim"], "rot_dim": s["latent_rot"],
+                                                   "vdim": s["latent_vdim"], "kv_rank": s["rank"],
+                                                   "scale": (s["latent_dim"] + s["latent_rot"]) ** -0.5,
+                                                   "rot": {"base": 10000.0, "dims": s["latent_rot"]}}, "mlp": mlp},
+            {"type": "rglru", "mixer": {"width": s["lru_width"], "blocks": s["lru_blocks"], "conv": s["taps"]}, "mlp": mlp},
+        ]
+    fadutar = {"architecture": "Fadutar", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5}, "layers": layers}
+    llama = dict(TINYLLAMA, hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=len(layers),
+                 num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], vocab_size=s["vocab"], max_position_embeddings=4096)
+    return fadutar, llama
+
+
+def bench_design(args, torch) -> int:
+    """`--design fadutar`: one JSON line.  Per size: tokens a second of a prompt step of 2048 tokens and of decode steps
+    at the record's batch and context, for the Fadutar decoder and for the Llama decoder of equal sizes (random
+    weights, bfloat16, through the engine's own loop), and every kernel the design adds alone, beside the like kernel."""
+    from tlie_amd import Engine, ops
+    from tlie_amd.kernel_bench import bench_design_kernels
+    peaks = ops.measured_peaks("cuda:0")
+    record = {"metric": f"{args.design}: prefill and decode tok/s beside the Llama decoder of equal sizes", "unit": "tokens/s",
+              "n_gpus": 1, "dtype": "bf16", "data": "synthetic: uniform random token ids, random weights",
+              "batch": args.batch, "context": args.context, "measured_peaks": peaks, "sizes": {}}
+    steps, warmup = min(args.steps, 48), 4
+    for name, sizes in DESIGN_SIZES.items():
+        entry = {"layers": 4 * sizes["groups"], "sizes": sizes}
+        for model, config in zip(("fadutar", "llama"), design_configs(sizes)):
+            engine = Engine(None, dtype="bfloat16", config=config, random_seed=0, max_tokens=args.batch * args.context + 4096,
+                            page_size=16, max_requests=args.batch + 1)
+            seconds = time_prefill(engine, torch, 2048, sizes["vocab"])
+            entry[f"{model}_prefill_2048_tok_s"] = 2048 / seconds
+            entry[f"{model}_prefill_2048_ms"] = seconds * 1e3
+            seconds = sorted(time_decode(engine, torch, args.batch, args.context, steps, warmup, sizes["vocab"]) for _ in range(3))[1]
+            entry[f"{model}_decode_tok_s"] = args.batch * steps / seconds
+            entry[f"{model}_decode_ms_step"] = seconds / steps * 1e3
+            del engine
+            torch.cuda.empty_cache()
+        entry["kernels"] = bench_design_kernels(sizes, batch=args.batch, context=args.context, prompt=2048,
+                                                hbm_gbs=peaks["stream_read_gbs"], mfma_tflops=peaks["mfma_bf16_tflops"])
+        record["sizes"][name] = entry
+    record["library_fallbacks"] = ops.library_fallbacks()
+    print(json.dumps(record))
+    return 0
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -186,6 +254,9 @@ def main() -> int:
                         help="time the kernels of a decode step (--batch, --context) and of a prompt step one by one at the "
                              "shape's layer sizes, each inside a replayed recording that walks through copies of its weights; "
                              "NAME keeps the kernels whose name holds it; prints one JSON line per kernel")
+    parser.add_argument("--design", default=None, choices=["fadutar"],
+                        help="prefill and decode throughput of that decoder design at layer sizes of real models, beside the Llama "
+                             "decoder at equal sizes, and its own kernels alone beside the like kernels (one JSON line of its own)")
     parser.add_argument("--shape", default="tinyllama", choices=["tinyllama", *OTHER_SHAPES],
                         help="layer sizes of another model of the same architecture (the default is the record's)")
     args = parser.parse_args()
@@ -194,6 +265,8 @@ def main() -> int:
         return 2
     import torch
     from tlie_amd import Engine
+    if args.design:
+        return bench_design(args, torch)
     cfg, model_name = dict(TINYLLAMA), "TinyLlama 1.1B shape"
     if args.shape != "tinyllama":
         model_name = OTHER_SHAPES[args.shape][0]

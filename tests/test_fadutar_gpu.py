@@ -227,13 +227,18 @@ def test_a_sink_that_is_left_out_and_a_key_past_the_chunk_edge_show():
     assert float(share[0]) < 0.03 < 0.9 < float(share[1])
 
 
-@pytest.mark.parametrize("width,blocks,taps", [(64, 1, 1), (48, 3, 5), (130, 2, 4)])
-def test_convolution_and_recurrence_carry_their_state(width, blocks, taps):
+SHORT_STEPS = ([23, 9], [(1, 4), (5, 0), (2, 1), (1, 1), (14, 3)])
+LONG_STEPS = ([300, 101], [(130, 1), (1, 70), (100, 0), (68, 29), (1, 1)])        # portions long enough for the sliced form
+
+
+@pytest.mark.parametrize("width,blocks,taps,plan", [(64, 1, 1, SHORT_STEPS), (48, 3, 5, SHORT_STEPS), (130, 2, 4, SHORT_STEPS),
+                                                    (48, 3, 5, LONG_STEPS), (130, 1, 2, LONG_STEPS)])
+def test_convolution_and_recurrence_carry_their_state(width, blocks, taps, plan):
     """Two sequences of unequal length in steps of unequal portions (down to one token), in slots that are
     not in order, against the plain functions on each whole sequence."""
     from tlie_amd import ops
     generator = torch.Generator().manual_seed(width)
-    lengths, slots = [23, 9], [2, 0]
+    (lengths, steps), slots = plan, [2, 0]
     inside = width // blocks
     conv, conv_bias = torch.randn(width, taps, generator=generator), torch.randn(width, generator=generator)
     gate_r, gate_i = (torch.randn(blocks, inside, inside, generator=generator) / math.sqrt(inside) for _ in range(2))
@@ -251,7 +256,7 @@ def test_convolution_and_recurrence_carry_their_state(width, blocks, taps):
     state[1] = 5.0                                                    # a slot that belongs to nobody stays as it is
     got = [[], []]
     at = [0, 0]
-    for step, counts in enumerate([(1, 4), (5, 0), (2, 1), (1, 1), (14, 3)]):
+    for step, counts in enumerate(steps):
         live = [s for s in (0, 1) if counts[s] > 0]
         rows = torch.cat([fused[s][at[s]:at[s] + counts[s]] for s in live]).to(DEVICE).contiguous()
         seq_start = torch.tensor([0] + list(torch.tensor([counts[s] for s in live]).cumsum(0)), dtype=torch.int32, device=DEVICE)
@@ -262,7 +267,8 @@ def test_convolution_and_recurrence_carry_their_state(width, blocks, taps):
         u = ops.causal_conv(product, width, conv.to(DEVICE), conv_bias.to(DEVICE), state, token_seq, token_slot, seq_start)
         gates = torch.empty(rows.shape[0], 2 * width, device=DEVICE)
         ops.block_linear(u, 0, width, inside, gates_t, gate_bias, gates, 0, 2 * width, 2 * inside, rows.shape[0])
-        out = ops.gated_recurrence(product, width, 0, u, gates, lam.to(DEVICE), 8.0, state, seq_start, seq_slot, inside, torch.float32)
+        out = ops.gated_recurrence(product, width, 0, u, gates, lam.to(DEVICE), 8.0, state, seq_start, seq_slot, inside, torch.float32,
+                                   max_new=max(counts))
         for i, s in enumerate(live):
             got[s].append(out[int(seq_start[i]):int(seq_start[i + 1])].cpu())
             at[s] += counts[s]
@@ -413,3 +419,21 @@ def test_a_preempted_request_is_recomputed_from_a_state_of_zero(setups):
     stats = {}
     assert engine.generate(prompts, max_tokens=20, stats=stats, admit_partial=True) == want
     engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_latent_attention_with_keys_wider_than_a_head_size(tmp_path, dtype):
+    """A latent vector and rotated part that together pass the widest head the attention kernels take: the
+    cache then keeps values of rank rows only and the plain kernel reads it."""
+    raw = {"architecture": "Fadutar", "vocab": 64, "width": 32, "norm": {"eps": 1e-5}, "layers": [
+        {"type": "latent_attention", "mixer": {"heads": 2, "dim": 8, "rot_dim": 12, "vdim": 8, "kv_rank": 250, "scale": 0.2,
+                                               "rot": {"base": 100.0, "dims": 12}}, "mlp": None}]}
+    folder = make_model(tmp_path, raw, seed=4)
+    config, weights = load_plain(folder)
+    tokens = tokens_of(8, 50, 64)
+    want = plain_forward(config, weights, tokens)
+    from tlie_amd import Engine
+    engine = Engine(folder, dtype=dtype, max_tokens=128, page_size=16, max_requests=2)
+    assert not engine.model.blocks[0].mixer.wide_values
+    for cuts in ([50], [1], [20, 3, 1]):
+        assert_rows(run_cut(engine, "a", tokens, cuts), want, TOLERANCE[dtype], f"cut {cuts}")

@@ -10,6 +10,9 @@
 // values.  The heads' own key and value matrices are applied to the queries before and to the attended
 // latent vectors after the attention (the block-diagonal products), which gives the same scores and
 // results as expanding every cached position's keys and values.
+// The value side of a page has `value_rows` rows of a page's positions: rank of them, or rank + rot when
+// the attention kernel that reads the page wants values as wide as keys; rows from rank on are never
+// written, and hold the zeros the pool was made with.
 //
 // Rotation: the pair (i, i + rot/2) by angle = float(position) * inv_freq[i], sines and cosines float.
 // Norm: c = x * rsqrt(mean(x^2) + eps) * weight over the rank dims, in float.
@@ -24,7 +27,7 @@ __global__ void latent_place_kernel(const D* __restrict__ fused, int nsplit, siz
                                     const int* __restrict__ positions, const int* __restrict__ slot_map,
                                     const float* __restrict__ inv_freq, const W* __restrict__ norm_weight, float eps,
                                     A* __restrict__ q_plain, A* __restrict__ q_wide, A* __restrict__ cache, int heads,
-                                    int plain, int rot, int rank, int page_size) {
+                                    int plain, int rot, int rank, int value_rows, int page_size) {
   extern __shared__ float lds[];
   const int half = rot / 2;
   float* cosines = lds;                  // half
@@ -49,7 +52,7 @@ __global__ void latent_place_kernel(const D* __restrict__ fused, int nsplit, siz
   };
   const int slot = slot_map[t];
   if (slot >= 0) {
-    A* page = cache + static_cast<size_t>(slot / page_size) * page_size * (key + rank);
+    A* page = cache + static_cast<size_t>(slot / page_size) * page_size * (key + value_rows);
     const int row = slot % page_size;
     for (int i = threadIdx.x; i < key; i += blockDim.x) {
       if (i < rank) {
@@ -77,9 +80,10 @@ using namespace tlie;
 extern "C" int tlie_latent_place(const void* fused, int in_dtype, int nsplit, long long split_stride, const int* positions,
                                  const int* slot_map, const float* inv_freq, const void* norm_weight, int weight_dtype,
                                  float eps, void* q_plain, void* q_wide, void* cache, int act_dtype, int tokens, int heads,
-                                 int plain, int rot, int rank, int page_size, void* stream) {
+                                 int plain, int rot, int rank, int value_rows, int page_size, void* stream) {
   if (tokens <= 0 || heads <= 0 || plain <= 0 || rot < 0 || rot % 2 != 0 || rank <= 0 || page_size <= 0 || nsplit < 1)
     return kBadArgument;
+  if (value_rows != rank && value_rows != rank + rot) return kBadArgument;
   if (rot > 0 && inv_freq == nullptr) return kBadArgument;
   const int widest = heads * (plain + rot);
   const int threads = widest >= 1024 ? 1024 : (widest >= 256 ? 256 : 64);
@@ -89,7 +93,7 @@ extern "C" int tlie_latent_place(const void* fused, int in_dtype, int nsplit, lo
   if (in_dtype == DC && weight_dtype == WC && act_dtype == AC) {                                                     \
     hipLaunchKernelGGL((latent_place_kernel<D, W, A>), dim3(tokens), dim3(threads), lds, s, (const D*)fused, nsplit,   \
                        (size_t)split_stride, positions, slot_map, inv_freq, (const W*)norm_weight, eps, (A*)q_plain,  \
-                       (A*)q_wide, (A*)cache, heads, plain, rot, rank, page_size);                                   \
+                       (A*)q_wide, (A*)cache, heads, plain, rot, rank, value_rows, page_size);                                   \
     return launch_status();                                                                                          \
   }
   TLIE_CASE(kF32, float, kF32, float, kF32, float)

@@ -14,6 +14,12 @@
 //
 // Tokens and sequences whose request slot is negative pad a recorded step: nothing is read or written
 // for them.
+//
+// A step that brings many tokens of a sequence takes the recurrence in slices of kSlice tokens: one
+// kernel leaves every slice's product of decays P and its end state E from a start of zero (and the
+// state the sequence came with), a second one gives every slice its carry, carry_z = P_(z-1) carry_(z-1) +
+// E_(z-1) from the sequence's state on, and walks the slice from there as the one-kernel form walks the
+// whole sequence.  The slices of a sequence then run side by side; the decays are computed twice.
 #include "common.h"
 
 namespace tlie {
@@ -23,6 +29,19 @@ __device__ __forceinline__ float softplus_f(float v) { return v > 20.f ? v : log
 __device__ __forceinline__ float gelu_tanh_f(float z) {
   return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
+
+// what token t does to channel c's state: S <- a * S + b
+__device__ __forceinline__ void decay_and_drive(const float* __restrict__ gates, const float* __restrict__ u, size_t t,
+                                                size_t gate_row, size_t gate_at, int block_width, int channels, int c,
+                                                float rate, float& a, float& b) {
+  const float r = sigmoid_f(gates[t * gate_row + gate_at]);
+  const float i = sigmoid_f(gates[t * gate_row + gate_at + block_width]);
+  const float log_a = rate * r;
+  a = expf(log_a);
+  b = sqrtf(-expm1f(2.f * log_a)) * (i * u[t * channels + c]);
+}
+
+constexpr int kSlice = 32;             // tokens of a slice in the sliced form
 
 // in: [nsplit][tokens][in_width], the convolution's inputs in columns x_col .. x_col + channels - 1.
 // u: [tokens][channels] float.  One thread a (token, channel).
@@ -56,7 +75,8 @@ __global__ void gated_recurrence_kernel(const D* __restrict__ in, int nsplit, si
                                         int y_col, const float* __restrict__ u, const float* __restrict__ gates,
                                         const W* __restrict__ lambda, float decay, float* __restrict__ state,
                                         const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
-                                        O* __restrict__ out, int channels, int block_width, int ntaps) {
+                                        O* __restrict__ out, int channels, int block_width, int ntaps,
+                                        const float* __restrict__ parts) {
   const int seq = blockIdx.x;
   const int slot = seq_slot[seq];
   if (slot < 0) return;
@@ -68,17 +88,30 @@ __global__ void gated_recurrence_kernel(const D* __restrict__ in, int nsplit, si
   const int block = c / block_width, inside = c % block_width;
   const size_t gate_row = static_cast<size_t>(channels) * 2, gate_at = static_cast<size_t>(block) * 2 * block_width + inside;
   const float rate = -decay * softplus_f(to_float(lambda[c]));
-  float s = held[static_cast<size_t>(ntaps - 1) * channels + c];
-  for (int k = 0; k < count; ++k) {
+  // slices == 0: the whole sequence in this thread, from and to the state.  Otherwise this thread takes slice
+  // blockIdx.z of its sequence, from the carry that the slices before it leave (`parts`, see below).
+  const int slices = parts != nullptr ? static_cast<int>(gridDim.z) : 0;
+  int begin = 0, end = count;
+  float s;
+  if (slices == 0) {
+    s = held[static_cast<size_t>(ntaps - 1) * channels + c];
+  } else {
+    begin = blockIdx.z * kSlice, end = min(count, begin + kSlice);
+    if (begin >= count) return;
+    const float* mine = parts + static_cast<size_t>(seq) * (2 * slices + 1) * channels;
+    s = mine[static_cast<size_t>(2 * slices) * channels + c];                    // the state the sequence came with
+    for (int z = 0; z < static_cast<int>(blockIdx.z); ++z)
+      s = mine[static_cast<size_t>(2 * z) * channels + c] * s + mine[static_cast<size_t>(2 * z + 1) * channels + c];
+  }
+  for (int k = begin; k < end; ++k) {
     const size_t t = static_cast<size_t>(first + k);
-    const float r = sigmoid_f(gates[t * gate_row + gate_at]);
-    const float i = sigmoid_f(gates[t * gate_row + gate_at + block_width]);
-    const float log_a = rate * r;
-    const float a = expf(log_a);
-    s = a * s + sqrtf(-expm1f(2.f * log_a)) * (i * u[t * channels + c]);
+    float a, b;
+    decay_and_drive(gates, u, t, gate_row, gate_at, block_width, channels, c, rate, a, b);
+    s = a * s + b;
     const float y = sum_splits(in + t * in_width + y_col + c, nsplit, split_stride);
     out[t * channels + c] = from_float<O>(s * gelu_tanh_f(y));
   }
+  if (end < count) return;                         // (only the sequence's last slice leaves the state)
   held[static_cast<size_t>(ntaps - 1) * channels + c] = s;
   // the last taps - 1 inputs of (what was held, then this step's): entry e of the new rows is entry
   // count + e of that sequence; rows are written in rising order and read at higher indices only
@@ -89,6 +122,40 @@ __global__ void gated_recurrence_kernel(const D* __restrict__ in, int nsplit, si
     else x = sum_splits(in + static_cast<size_t>(first + from - (ntaps - 1)) * in_width + x_col + c, nsplit, split_stride);
     held[static_cast<size_t>(e) * channels + c] = x;
   }
+}
+
+// parts: [sequences][2 * slices + 1][channels]: for slice z the product of its decays at 2z and its end state
+// from a start of zero at 2z + 1 (the last slice of a sequence leaves none: nobody reads it); at 2 * slices the
+// state the sequence came with (the kernel above reads it from here, since its last slice writes the state
+// while other slices may still want the old one).
+__global__ void recurrence_slices_kernel(const float* __restrict__ u, const float* __restrict__ gates, const void* __restrict__ lambda,
+                                         int lambda_is_bf16, float decay, const float* __restrict__ state,
+                                         const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
+                                         float* __restrict__ parts, int channels, int block_width, int ntaps) {
+  const int seq = blockIdx.x, slices = gridDim.z;
+  const int slot = seq_slot[seq];
+  if (slot < 0) return;
+  const int first = seq_start[seq], count = seq_start[seq + 1] - first;
+  const int begin = blockIdx.z * kSlice, end = min(count, begin + kSlice);
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= channels || count <= 0) return;
+  float* mine = parts + static_cast<size_t>(seq) * (2 * slices + 1) * channels;
+  if (blockIdx.z == 0)
+    mine[static_cast<size_t>(2 * slices) * channels + c] = state[(static_cast<size_t>(slot) * ntaps + ntaps - 1) * channels + c];
+  if (end >= count) return;                        // past the sequence, or its last slice
+  const int block = c / block_width, inside = c % block_width;
+  const size_t gate_row = static_cast<size_t>(channels) * 2, gate_at = static_cast<size_t>(block) * 2 * block_width + inside;
+  const float lam = lambda_is_bf16 ? to_float(static_cast<const bf16*>(lambda)[c]) : static_cast<const float*>(lambda)[c];
+  const float rate = -decay * softplus_f(lam);
+  float product = 1.f, s = 0.f;
+  for (int k = begin; k < end; ++k) {
+    float a, b;
+    decay_and_drive(gates, u, static_cast<size_t>(first + k), gate_row, gate_at, block_width, channels, c, rate, a, b);
+    s = a * s + b;
+    product *= a;
+  }
+  mine[static_cast<size_t>(2 * blockIdx.z) * channels + c] = product;
+  mine[static_cast<size_t>(2 * blockIdx.z + 1) * channels + c] = s;
 }
 
 }  // namespace tlie
@@ -123,17 +190,27 @@ extern "C" int tlie_gated_recurrence(const void* in, int in_dtype, int nsplit, l
                                      int x_col, int y_col, const float* u, const float* gates, const void* lambda,
                                      int weight_dtype, float decay, float* state, const int* seq_start, const int* seq_slot,
                                      void* out, int out_dtype, int seqs, int channels, int block_width, int ntaps,
-                                     void* stream) {
+                                     int slices, float* parts, void* stream) {
+  // slices 0: a thread walks all of a sequence's tokens of the step.  slices > 0 (then no sequence brings more than
+  // slices * 32 tokens, and parts holds seqs * (2 * slices + 1) * channels floats): the sliced form.
+  if (slices < 0 || slices > 65535 || (slices > 0 && parts == nullptr)) return kBadArgument;
   if (seqs <= 0 || channels <= 0 || ntaps <= 0 || nsplit < 1 || block_width <= 0 || channels % block_width != 0) return kBadArgument;
   if (x_col < 0 || x_col + channels > in_width || y_col < 0 || y_col + channels > in_width) return kBadArgument;
-  const dim3 grid(seqs, (channels + 63) / 64);
+  const dim3 grid(seqs, (channels + 63) / 64, slices > 0 ? slices : 1);
   if (grid.y > 65535) return kBadArgument;
   hipStream_t s = (hipStream_t)stream;
+  if (slices > 0) {
+    if (weight_dtype != kF32 && weight_dtype != kBF16) return kBadArgument;
+    hipLaunchKernelGGL(recurrence_slices_kernel, grid, dim3(64), 0, s, u, gates, lambda, weight_dtype == kBF16 ? 1 : 0, decay,
+                       state, seq_start, seq_slot, parts, channels, block_width, ntaps);
+    if (launch_status() != kOk) return kLaunchFailed;
+  }
+  const float* carried = slices > 0 ? parts : nullptr;
 #define TLIE_CASE(DC, D, WC, W, OC, O)                                                                            \
   if (in_dtype == DC && weight_dtype == WC && out_dtype == OC) {                                                   \
     hipLaunchKernelGGL((gated_recurrence_kernel<D, W, O>), grid, dim3(64), 0, s, (const D*)in, nsplit,              \
                        (size_t)split_stride, in_width, x_col, y_col, u, gates, (const W*)lambda, decay, state,     \
-                       seq_start, seq_slot, (O*)out, channels, block_width, ntaps);                                \
+                       seq_start, seq_slot, (O*)out, channels, block_width, ntaps, carried);                       \
     return launch_status();                                                                                        \
   }
   TLIE_CASE(kF32, float, kF32, float, kF32, float)

@@ -199,3 +199,142 @@ def bench_kernels(cfg: dict, batch: int = 8, context: int = 2048, prompt: int = 
                              _timed(lambda i: ops.rope_cache(qkv, positions_p, positions_p, inv_freq, d, cache_p, nq, nkv, d, bf, paired=True),
                                     4, samples), read_bytes=prompt * (nq + 2 * nkv) * d * 4))
     return rows
+
+
+def bench_design_kernels(sizes: dict, batch: int = 8, context: int = 2048, prompt: int = 2048, samples: int = 10, device="cuda:0",
+                         hbm_gbs: float = 8000.0, mfma_tflops: float = 2500.0) -> list[dict]:
+    """The kernels that the Fadutar decoder adds, each alone at a layer's sizes, for a decode step of `batch`
+    requests at `context` positions and a prompt step of `prompt` tokens, each beside the like kernel of the
+    Llama decoder at the same sizes; every row carries the fraction of the roofline its bytes or flops reach
+    (`frac`: of `hbm_gbs` for rows with bytes, of `mfma_tflops` for rows with flops).
+    sizes: width, ff, heads, kv_heads, dim (attention, keys and values alike), chunk; latent_heads, latent_dim,
+    latent_rot, latent_vdim, rank; lru_width, lru_blocks, taps."""
+    device = torch.device(device)
+    torch.cuda.set_device(device)
+    bf, f32 = torch.bfloat16, torch.float32
+    width, ff = sizes["width"], sizes["ff"]
+    nq, nkv, d, chunk = sizes["heads"], sizes["kv_heads"], sizes["dim"], sizes["chunk"]
+    lh, ldim, lrot, lv, rank = sizes["latent_heads"], sizes["latent_dim"], sizes["latent_rot"], sizes["latent_vdim"], sizes["rank"]
+    lru, lru_blocks, taps = sizes["lru_width"], sizes["lru_blocks"], sizes["taps"]
+    page_size, rows = 16, []
+    units = int(torch.cuda.get_device_properties(device).multi_processor_count)
+
+    def rand(*shape, scale=0.02, dtype=bf):
+        return (torch.randn(shape, device=device, dtype=f32) * scale).to(dtype)
+
+    def row(name, times, read_bytes=0, flops=0):
+        entry = _row(name, times, read_bytes, flops)
+        if read_bytes:
+            entry["frac"] = round(entry["gbs"] / hbm_gbs, 3)
+        elif flops:
+            entry["frac"] = round(entry["tflops"] / mfma_tflops, 4)
+        rows.append(entry)
+
+    def ints(values):
+        return torch.tensor(values, dtype=torch.int32, device=device)
+
+    for label, tokens, seqs in ((f"decode b{batch}", batch, batch), (f"prompt {prompt}", prompt, 1)):
+        if tokens <= 0:
+            continue
+        decode = seqs == tokens
+        length = context if decode else prompt
+        blocks = (length + page_size - 1) // page_size
+        table = torch.arange(seqs * blocks, dtype=torch.int32, device=device).view(seqs, blocks).contiguous()
+        if decode:
+            positions = torch.full((tokens,), length - 1, dtype=torch.int32, device=device)
+            token_seq, seq_start = ints(list(range(tokens))), ints(list(range(tokens + 1)))
+            host = {"seq_start": np.arange(tokens + 1, dtype=np.int32), "seq_len": np.full(tokens, length, dtype=np.int32)}
+        else:
+            positions = torch.arange(tokens, dtype=torch.int32, device=device)
+            token_seq, seq_start = torch.zeros(tokens, dtype=torch.int32, device=device), ints([0, tokens])
+            host = {"seq_start": np.asarray([0, tokens], dtype=np.int32), "seq_len": np.asarray([tokens], dtype=np.int32)}
+        slot_map = (table[token_seq.long(), (positions // page_size).long()] * page_size + positions % page_size).to(torch.int32).contiguous()
+        seq_slot = ints(list(range(seqs)))
+        token_slot = seq_slot[token_seq.long()].contiguous()
+        ctx = SimpleNamespace(max_new=1 if decode else tokens, num_seqs=seqs, num_tokens=tokens, max_context=length, scratch={},
+                              tile_owner=None, compute_units=units, host=host, tokens=positions)
+        seen = min(length, chunk) if chunk else length            # keys a token of the chunked layers reads at most
+        # ---- attention with a sink inside chunks, on the matrix cores, beside the plain causal one --------------
+        cache = rand(seqs * blocks, 2, nkv, page_size * d, scale=0.5)
+        q = rand(tokens, nq * d, scale=1.0)
+        sink = rand(nq, scale=1.0, dtype=f32)
+        tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, nq // nkv, nkv, d)
+        for name, extra, keys in (("attention, causal (Llama's)", {}, length), (f"attention, sink + chunks of {chunk}", {"chunk": chunk, "sink": sink}, seen)):
+            launch = lambda i: ops.attention_mfma(q, cache, table, tiles, positions, nq, nkv, d, None, d ** -0.5, nsplit, split_len,
+                                                  col_tiles, waves, shared, **extra)
+            if decode:
+                row(f"{label}: {name}", _timed(launch, 4, samples), read_bytes=seqs * keys * 2 * nkv * d * 2)
+            else:
+                pairs = sum(p % chunk + 1 for p in range(tokens)) if extra and chunk else tokens * (tokens + 1) // 2
+                row(f"{label}: {name}", _timed(launch, 4, samples), flops=4.0 * nq * d * pairs)
+        # ---- latent attention: placement, the heads' products before and after, the attention over the latent cache ----
+        key = rank + lrot
+        fused = ops.Product(rand(tokens, lh * (ldim + lrot) + rank + lrot, scale=1.0), 1)
+        latent_cache = rand(seqs * blocks, 2, 1, page_size * key, scale=0.5)       # values as wide as keys
+        inv_freq = torch.pow(torch.tensor(10000.0), -2.0 * torch.arange(lrot // 2, dtype=f32) / lrot).to(device)
+        norm_weight = rand(rank, scale=1.0)
+        launch = lambda i: ops.latent_place(fused, positions, slot_map, inv_freq, norm_weight, 1e-5, latent_cache, lh, ldim, lrot, rank, bf,
+                                            wide_values=True)
+        row(f"{label}: latent placement (norm, rotation, cache write)", _timed(launch, 4, samples),
+            read_bytes=tokens * (fused.cols * 2 + lh * (ldim + lrot) * 2 + (key + rank) * 2))
+        q_plain, q_wide = launch(0)
+        up_keys, up_values = rand(lh, ldim, rank), rand(lh, rank, lv)
+        launch = lambda i: ops.block_linear(q_plain, 0, lh * ldim, ldim, up_keys, None, q_wide, 0, lh * key, key, tokens)
+        row(f"{label}: heads' queries onto the latent space [{lh} x {ldim} x {rank}]", _timed(launch, 4, samples),
+            **({"read_bytes": lh * ldim * rank * 2 + tokens * lh * (ldim + rank) * 2} if decode else {"flops": 2.0 * tokens * lh * ldim * rank}))
+        latent_sink = rand(lh, scale=1.0, dtype=f32)
+        ltiles, lcol_tiles, lnsplit, lsplit_len, lwaves, lshared = ops.attention_plan(ctx, lh, 1, key)
+        launch = lambda i: ops.attention_mfma(q_wide, latent_cache, table, ltiles, positions, lh, 1, key, None, 0.1, lnsplit, lsplit_len,
+                                              lcol_tiles, lwaves, lshared, sink=latent_sink)
+        if decode:
+            row(f"{label}: attention over the latent cache ({lh} heads, {key} key dims)", _timed(launch, 4, samples),
+                read_bytes=seqs * length * (key + rank) * 2)
+        else:
+            row(f"{label}: attention over the latent cache ({lh} heads, {key} key dims)", _timed(launch, 2, samples),
+                flops=2.0 * lh * (key + rank) * tokens * (tokens + 1) / 2)
+        attended = rand(tokens, lh * key, scale=1.0)
+        values = torch.empty((tokens, lh * lv), dtype=bf, device=device)
+        launch = lambda i: ops.block_linear(attended, 0, lh * key, key, up_values, None, values, 0, lh * lv, lv, tokens)
+        row(f"{label}: attended latent vectors onto the heads' values [{lh} x {rank} x {lv}]", _timed(launch, 4, samples),
+            **({"read_bytes": lh * rank * lv * 2 + tokens * lh * (rank + lv) * 2} if decode else {"flops": 2.0 * tokens * lh * rank * lv}))
+        # ---- the recurrence: convolution, gates, scan -------------------------------------------------------------
+        inside = lru // lru_blocks
+        both = ops.Product(rand(tokens, 2 * lru, scale=1.0), 1)
+        state = torch.zeros((seqs, taps, lru), dtype=f32, device=device)
+        conv, conv_bias = rand(lru, taps, scale=0.5), rand(lru)
+        launch = lambda i: ops.causal_conv(both, lru, conv, conv_bias, state, token_seq, token_slot, seq_start)
+        row(f"{label}: causal convolution [{lru} x {taps}]", _timed(launch, 4, samples), read_bytes=tokens * lru * (2 + 4) + seqs * taps * lru * 4)
+        u = launch(0)
+        gates_t, gate_bias = rand(lru_blocks, inside, 2 * inside), rand(lru_blocks, 2 * inside)
+        gates = torch.empty((tokens, 2 * lru), dtype=f32, device=device)
+        launch = lambda i: ops.block_linear(u, 0, lru, inside, gates_t, gate_bias, gates, 0, 2 * lru, 2 * inside, tokens)
+        row(f"{label}: the recurrence's gates [{lru_blocks} x {inside} x {2 * inside}]", _timed(launch, 4, samples),
+            **({"read_bytes": lru_blocks * inside * 2 * inside * 2 + tokens * lru * 12} if decode else {"flops": 4.0 * tokens * lru * inside}))
+        lam = rand(lru, scale=1.0)
+        launch = lambda i: ops.gated_recurrence(both, lru, 0, u, gates, lam, 8.0, state, seq_start, seq_slot, inside, bf, max_new=ctx.max_new)
+        row(f"{label}: gated recurrence (scan, gate branch, state)", _timed(launch, 4, samples),
+            read_bytes=tokens * lru * (4 + 8 + 4 + 2) + seqs * taps * lru * 8)
+        # ---- the element-wise kernels beside Llama's ------------------------------------------------------------------
+        residual = rand(tokens, width, scale=1.0, dtype=f32)
+        delta = ops.Product(rand(tokens, width, scale=1.0), 1)
+        weight, weight32 = rand(width, scale=1.0), rand(width, scale=1.0, dtype=f32)
+        row(f"{label}: add + norm (Llama's) [{tokens} x {width}]",
+            _timed(lambda i: ops.add_rmsnorm(residual, delta, weight, 1e-5, bf), 4, samples), read_bytes=tokens * width * (4 + 2 + 4 + 2))
+        row(f"{label}: norm + add + norm [{tokens} x {width}]",
+            _timed(lambda i: ops.norm_add_rmsnorm(residual, delta, weight32, 1e-5, weight32, 1e-5, bf), 4, samples),
+            read_bytes=tokens * width * (4 + 2 + 4 + 2))
+        gate_up = ops.Product(rand(tokens, 2 * ff, scale=1.0), 1)
+        row(f"{label}: silu gate (Llama's) [{tokens} x {ff}]", _timed(lambda i: ops.silu_mul(gate_up, bf, interleaved=True), 4, samples),
+            read_bytes=tokens * ff * 6)
+        row(f"{label}: clamped gate [{tokens} x {ff}]",
+            _timed(lambda i: ops.silu_mul(gate_up, bf, interleaved=True, gate="clamped_swish", alpha=1.702, limit=7.0), 4, samples),
+            read_bytes=tokens * ff * 6)
+        qkv = ops.Product(rand(tokens, (nq + 2 * nkv) * d, scale=1.0), 1)
+        rot_freq = torch.pow(torch.tensor(10000.0), -2.0 * torch.arange(d // 2, dtype=f32) / d).to(device)
+        row(f"{label}: rotation + cache write (Llama's)",
+            _timed(lambda i: ops.rope_cache(qkv, positions, slot_map, rot_freq, d, cache, nq, nkv, d, bf, paired=True), 4, samples),
+            read_bytes=tokens * (nq + 2 * nkv) * d * 4)
+        row(f"{label}: placement of q, k, v (no rotation)",
+            _timed(lambda i: ops.qkv_place(qkv, positions, slot_map, None, 0, cache, nq, nkv, d, d, bf), 4, samples),
+            read_bytes=tokens * (nq + 2 * nkv) * d * 4)
+    return rows

@@ -422,12 +422,15 @@ def block_linear(x: torch.Tensor, x_offset: int, x_row: int, x_block: int, weigh
 
 def latent_place(fused: Product, positions: torch.Tensor, slot_map: torch.Tensor, inv_freq: torch.Tensor | None,
                  norm_weight: torch.Tensor, eps: float, cache: torch.Tensor, heads: int, plain: int, rot: int, rank: int,
-                 act_dtype: torch.dtype) -> tuple[torch.Tensor, torch.Tensor]:
+                 act_dtype: torch.dtype, wide_values: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
     """Latent attention between its first product and the attention kernel.  fused: [T, heads * (plain +
     rot) + rank + rot].  The rank dims are RMS-normed (weight, eps) and written to the cache rows of
     `slot_map` as keys [row][rank + rot] beside the rotated shared key part, and once more, transposed, as
     values; returns (q_plain [T, heads * plain], q_wide [T, heads, rank + rot] of which only each head's
-    last rot dims, the rotated ones, are filled: the per-head product of q_plain fills the rest)."""
+    last rot dims, the rotated ones, are filled: the per-head product of q_plain fills the rest).
+    wide_values: the value side of a page has rank + rot rows, as many as a key has dims (the cache is then
+    [pages, 2, 1, page_size * (rank + rot)], what an attention kernel with one head size reads); its last rot
+    rows are never written."""
     _check_product(fused, "fused")
     _device_tensor(positions, "positions", torch.int32)
     _device_tensor(slot_map, "slot_map", torch.int32)
@@ -444,14 +447,14 @@ def latent_place(fused: Product, positions: torch.Tensor, slot_map: torch.Tensor
         _device_tensor(inv_freq, "inv_freq", torch.float32)
     if not eps > 0.0:
         raise EngineError(ErrorCode.NUMERICAL, "RMSNorm requires a positive epsilon")
-    page_size = _check_cache(cache, 1, rank + rot, "latent_place", rank)
+    page_size = _check_cache(cache, 1, rank + rot, "latent_place", rank + rot if wide_values else rank)
     q_plain = torch.empty((tokens, heads * plain), dtype=act_dtype, device=cache.device)
     q_wide = torch.empty((tokens, heads * (rank + rot)), dtype=act_dtype, device=cache.device)
     _check(library().tlie_latent_place(_ptr(fused.data), dtype_code(fused.data.dtype), fused.nsplit,
                                        ctypes.c_longlong(fused.split_stride), _ptr(positions), _ptr(slot_map), _ptr(inv_freq),
                                        _ptr(norm_weight), dtype_code(norm_weight.dtype), ctypes.c_float(eps), _ptr(q_plain),
                                        _ptr(q_wide), _ptr(cache), dtype_code(act_dtype), tokens, heads, plain, rot, rank,
-                                       page_size, _stream()), "latent_place")
+                                       rank + rot if wide_values else rank, page_size, _stream()), "latent_place")
     return q_plain, q_wide
 
 
@@ -486,14 +489,21 @@ def causal_conv(fused: Product, x_col: int, taps: torch.Tensor, bias: torch.Tens
     return u
 
 
+RECURRENCE_SLICE = 32          # tokens of a slice of the sliced recurrence (the kernel's kSlice)
+RECURRENCE_SLICED_FROM = 64    # tokens a sequence brings from which the sliced form pays (three launches' worth of work)
+
+
 def gated_recurrence(fused: Product, x_col: int, y_col: int, u: torch.Tensor, gates: torch.Tensor, lam: torch.Tensor,
                      decay: float, state: torch.Tensor, seq_start: torch.Tensor, seq_slot: torch.Tensor, block_width: int,
-                     out_dtype: torch.dtype) -> torch.Tensor:
+                     out_dtype: torch.dtype, max_new: int = 1) -> torch.Tensor:
     """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t with a_t = exp(-decay * r_t * softplus(lam)), r and i the
     sigmoids of `gates` [T, blocks, 2 * block_width] (a block's r before its i), per channel and sequence,
     from and to row n-1 of state [slots, n, channels]; out = S * gelu_tanh(y), y in columns y_col .. of
     `fused`; the state's other rows get the step's last inputs of the convolution (columns x_col ..).
-    Sequences whose slot is negative are skipped."""
+    Sequences whose slot is negative are skipped.  max_new: the most tokens any sequence brings in this step
+    (the caller knows it on the host); beyond RECURRENCE_SLICED_FROM the sequences' tokens are taken in slices
+    that run side by side (each from the carry that the slices before it leave), else a thread walks a
+    sequence's tokens in order."""
     _check_product(fused, "fused")
     _device_tensor(u, "u", torch.float32)
     _device_tensor(gates, "gates", torch.float32)
@@ -509,11 +519,15 @@ def gated_recurrence(fused: Product, x_col: int, y_col: int, u: torch.Tensor, ga
     if not (0 <= x_col <= fused.cols - channels and 0 <= y_col <= fused.cols - channels):
         raise invalid_shape("gated_recurrence: the columns do not fit the product")
     out = torch.empty((tokens, channels), dtype=out_dtype, device=u.device)
+    slices, parts = 0, None
+    if max_new > RECURRENCE_SLICED_FROM:
+        slices = (min(int(max_new), tokens) + RECURRENCE_SLICE - 1) // RECURRENCE_SLICE
+        parts = torch.empty((seqs, 2 * slices + 1, channels), dtype=torch.float32, device=u.device)
     _check(library().tlie_gated_recurrence(_ptr(fused.data), dtype_code(fused.data.dtype), fused.nsplit,
                                            ctypes.c_longlong(fused.split_stride), fused.cols, x_col, y_col, _ptr(u), _ptr(gates),
                                            _ptr(lam), dtype_code(lam.dtype), ctypes.c_float(decay), _ptr(state), _ptr(seq_start),
                                            _ptr(seq_slot), _ptr(out), dtype_code(out_dtype), seqs, channels, block_width,
-                                           state.shape[1], _stream()), "gated_recurrence")
+                                           state.shape[1], slices, _ptr(parts), _stream()), "gated_recurrence")
     return out
 
 

@@ -11,6 +11,10 @@ taken to the latent space before the attention (one small product per head), the
 single key head of rank + rot dims whose values are the c themselves, and W_uv is applied per head to the
 attended latent vector afterwards: the same sums in another order, and no key or value is ever expanded
 for a cached position.  A page holds the rows [c | r] and, for the value side, c once more, transposed.
+While a key has no more dims than the attention kernels take as a head size, the value side is as wide as
+the key side (its last rot rows are never written and stay zero): the cache is then that of one key head
+of rank + rot dims, in bfloat16 the kernel on the matrix cores reads it (all heads' columns of a token share
+each read of a key), and the attended vector's first rank dims are what goes on.
 """
 from __future__ import annotations
 
@@ -56,6 +60,8 @@ class LatentAttention(Mixer):
         if self.rank > ops.ATTENTION_MAX_HEAD_DIM:
             raise invalid_config(f"latent_attention: a latent vector of {self.rank} dims is beyond the attention kernel's "
                                  f"{ops.ATTENTION_MAX_HEAD_DIM} value dims")
+        # values as wide as keys while that is a head size the attention kernels take
+        self.wide_values = self.rank + self.rot <= ops.ATTENTION_MAX_HEAD_DIM
         self.inv_freq = None
         if self.rot > 0:
             position = spec["position"]
@@ -96,7 +102,10 @@ class LatentAttention(Mixer):
             self.sink = keep(weights[prefix + names["sink"]].float().contiguous())
 
     def cache_need(self):
-        """One key head of rank + rot dims, [row][dim], then its rank value dims transposed, [dim][row]."""
+        """One key head of rank + rot dims, [row][dim], then its value dims transposed, [dim][row]: rank of them, or
+        with wide values as many as a key has."""
+        if self.wide_values:
+            return CacheNeed((2, 1), self.rank + self.rot, None)
         return CacheNeed((1,), 2 * self.rank + self.rot, None)
 
     def forward(self, x, ctx, binding: Binding, into=None):
@@ -106,13 +115,20 @@ class LatentAttention(Mixer):
         tokens = fused.rows
         q_plain, q_wide = ops.latent_place(fused, ctx.positions, pages.slot_map if binding.writes else ctx.no_slots, self.inv_freq,
                                            self.down_norm, self.norm_eps, binding.cache, self.heads, self.plain, self.rot,
-                                           self.rank, self.dtype)
+                                           self.rank, self.dtype, wide_values=self.wide_values)
         ops.block_linear(q_plain, 0, self.heads * self.plain, self.plain, self.up_keys, None,
                          q_wide, 0, self.heads * key, key, tokens)
-        attended = ops.attention_generic(q_wide, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.heads, 1,
-                                         key, None, self.scale, tiled=ops.attention_generic_plan(ctx, key, self.rank),
-                                         seq_start=ctx.seq_start, value_dim=self.rank, sink=self.sink)
+        value_dim = key if self.wide_values else self.rank
+        if self.wide_values and ops.attention_mfma_takes(self.dtype, key, binding.cache.shape[-1] // key):
+            tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, self.heads, 1, key)
+            attended = ops.attention_mfma(q_wide, binding.cache, pages.block_table, tiles, ctx.positions, self.heads, 1, key,
+                                          None, self.scale, nsplit, split_len, col_tiles, waves, shared, sink=self.sink)
+        else:
+            attended = ops.attention_generic(q_wide, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.heads, 1,
+                                             key, None, self.scale, tiled=ops.attention_generic_plan(ctx, key, value_dim),
+                                             seq_start=ctx.seq_start, value_dim=value_dim, sink=self.sink)
+        # (of every head's attended vector the first rank dims: with wide values the rest are zeros)
         values = torch.empty((tokens, self.heads * self.dv), dtype=self.dtype, device=attended.device)
-        ops.block_linear(attended, 0, self.heads * self.rank, self.rank, self.up_values_t, None,
+        ops.block_linear(attended, 0, self.heads * value_dim, value_dim, self.up_values_t, None,
                          values, 0, self.heads * self.dv, self.dv, tokens)
         return self.o(values)

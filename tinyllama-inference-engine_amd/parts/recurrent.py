@@ -94,5 +94,5 @@ class GatedRecurrence(Mixer):
         ops.block_linear(u, 0, width, self.block_width, self.gates_t, self.gate_bias,
                          gates, 0, 2 * width, 2 * self.block_width, tokens)
         mixed = ops.gated_recurrence(fused, width, 0, u, gates, self.lam, self.decay, binding.state, ctx.seq_start, ctx.seq_slot,
-                                     self.block_width, self.dtype)
+                                     self.block_width, self.dtype, max_new=ctx.max_new)
         return self.o(mixed)
