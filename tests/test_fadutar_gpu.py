@@ -107,6 +107,29 @@ def test_block_diagonal_product(rows, blocks, inner, outer):
     assert float((out[:, :, 0] - 7.0).abs().max()) == 0.0 and float((out[:, :, 1 + outer:] - 7.0).abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("rows,blocks,inner,outer,wide", [(17, 3, 32, 16, False), (200, 2, 96, 70, True), (129, 5, 64, 3, False), (300, 1, 256, 512, True)])
+def test_block_diagonal_product_on_the_matrix_cores(rows, blocks, inner, outer, wide):
+    """bfloat16 weights, x in bfloat16 or (wide) in float, many rows: against float64 on the same rounded operands."""
+    from tlie_amd import ops
+    generator = torch.Generator().manual_seed(rows + inner)
+    x_wide, out_wide = inner + 8, outer + 3
+    x = torch.randn(rows, blocks, x_wide, generator=generator).bfloat16()
+    weight = (torch.randn(blocks, outer, inner, generator=generator) / inner ** 0.5).bfloat16()
+    bias = torch.randn(blocks, outer, generator=generator).bfloat16()
+    want = torch.einsum("tbi,boi->tbo", x[:, :, 8:8 + inner].double(), weight.double()) + bias.double()
+    given = (x.float() if wide else x).to(DEVICE)
+    out = torch.full((rows, blocks, out_wide), 7.0, device=DEVICE, dtype=torch.float32)
+    ops.block_linear(given, 8, blocks * x_wide, x_wide, weight.transpose(1, 2).contiguous().to(DEVICE), bias.to(DEVICE),
+                     out, 1, blocks * out_wide, out_wide, rows, weight=weight.to(DEVICE))
+    assert float((out[:, :, 1:1 + outer].cpu().double() - want).abs().max()) < 1e-4
+    assert float((out[:, :, 0] - 7.0).abs().max()) == 0.0 and float((out[:, :, 1 + outer:] - 7.0).abs().max()) == 0.0
+    # and the same rows through the plain kernel: the two routes agree to the sums' rounding
+    plain = torch.full((rows, blocks, out_wide), 7.0, device=DEVICE, dtype=torch.float32)
+    ops.block_linear(given, 8, blocks * x_wide, x_wide, weight.transpose(1, 2).contiguous().to(DEVICE), bias.to(DEVICE),
+                     plain, 1, blocks * out_wide, out_wide, rows)
+    assert float((out - plain).abs().max()) < 1e-4
+
+
 def _attend(q, k, v, sink, scale, chunk, page_size, cuts, dtype=torch.float32):
     """q [T, H, d], k [T, G, d], v [T, G, dv] of one sequence through the placing kernel and the attention
     kernel, in steps of the sizes `cuts`, with the sequence's pages in a scrambled order."""

@@ -53,9 +53,104 @@ block_linear_kernel(const X* __restrict__ x, long long x_row, long long x_block,
   }
 }
 
+// The same product on the matrix cores, for steps of many rows: bfloat16 weights kept as they are stored,
+// [blocks][outer][inner]; x bfloat16, or float that is rounded to bfloat16 as it becomes an operand; float
+// sums.  A wave takes 32 rows of x and 64 outputs of one block, a workgroup of four waves 128 rows: every
+// operand goes from memory (the weights of a block are small: from the caches) straight into the registers
+// of v_mfma_f32_16x16x32_bf16, whose A operand is 16 rows of the weight (a lane: row lane % 16, 8 inner values
+// from (lane / 16) * 8 on) and whose B operand is 16 rows of x laid out alike; a lane then holds 4 consecutive
+// outputs of one row of x.  inner % 32 == 0, and all offsets and strides of x multiples of 8 elements.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
+
+__device__ __forceinline__ bf16x8_t operand_of(const bf16* p) { return *reinterpret_cast<const bf16x8_t*>(p); }
+__device__ __forceinline__ bf16x8_t operand_of(const float* p) {
+  const float4 lo = *reinterpret_cast<const float4*>(p), hi = *reinterpret_cast<const float4*>(p + 4);
+  union { uint32_t w[4]; bf16x8_t v; } packed;
+  packed.w[0] = pack_bf16(lo.x, lo.y), packed.w[1] = pack_bf16(lo.z, lo.w);
+  packed.w[2] = pack_bf16(hi.x, hi.y), packed.w[3] = pack_bf16(hi.z, hi.w);
+  return packed.v;
+}
+
+template <typename X, typename Y>
+__global__ void __launch_bounds__(256)
+block_linear_mfma_kernel(const X* __restrict__ x, long long x_row, long long x_block, const bf16* __restrict__ w,
+                         const bf16* __restrict__ bias, Y* __restrict__ y, long long y_row, long long y_block, int rows,
+                         int inner, int outer) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, grp = lane >> 4;
+  const int b = blockIdx.y, row0 = blockIdx.x * 128 + wave * 32, out0 = blockIdx.z * 64;
+  if (row0 >= rows) return;                        // (the whole wave)
+  // rows and outputs past the end are read from the last one and not stored
+  const X* x_at[2];
+  const bf16* w_at[4];
+#pragma unroll
+  for (int r = 0; r < 2; ++r)
+    x_at[r] = x + static_cast<size_t>(min(row0 + r * 16 + col, rows - 1)) * x_row + static_cast<size_t>(b) * x_block + grp * 8;
+#pragma unroll
+  for (int o = 0; o < 4; ++o)
+    w_at[o] = w + (static_cast<size_t>(b) * outer + min(out0 + o * 16 + col, outer - 1)) * inner + grp * 8;
+  floatx4_t acc[2][4];
+#pragma unroll
+  for (int r = 0; r < 2; ++r)
+#pragma unroll
+    for (int o = 0; o < 4; ++o) acc[r][o] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k = 0; k < inner; k += 32) {
+    bf16x8_t from_x[2], from_w[4];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) from_x[r] = operand_of(x_at[r] + k);
+#pragma unroll
+    for (int o = 0; o < 4; ++o) from_w[o] = operand_of(w_at[o] + k);
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+      for (int o = 0; o < 4; ++o) acc[r][o] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(from_w[o], from_x[r], acc[r][o], 0, 0, 0);
+  }
+  // acc[r][o][j] is output out0 + o * 16 + grp * 4 + j of row row0 + r * 16 + col
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int row = row0 + r * 16 + col;
+    if (row >= rows) continue;
+#pragma unroll
+    for (int o = 0; o < 4; ++o)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int out = out0 + o * 16 + grp * 4 + j;
+        if (out < outer) {
+          const float shift = bias != nullptr ? to_float(bias[static_cast<size_t>(b) * outer + out]) : 0.f;
+          y[static_cast<size_t>(row) * y_row + static_cast<size_t>(b) * y_block + out] = from_float<Y>(acc[r][o][j] + shift);
+        }
+      }
+  }
+}
+
 }  // namespace tlie
 
 using namespace tlie;
+
+// w: bfloat16 [blocks][outer][inner] (as stored: [out, in] per block); otherwise as tlie_block_linear.
+extern "C" int tlie_block_linear_mfma(const void* x, int x_dtype, long long x_row, long long x_block, const void* w,
+                                      const void* bias, void* y, int y_dtype, long long y_row, long long y_block, int rows,
+                                      int blocks, int inner, int outer, void* stream) {
+  if (rows <= 0 || blocks <= 0 || blocks > 65535 || inner <= 0 || inner % 32 != 0 || outer <= 0) return kBadArgument;
+  if (x_row % 8 != 0 || x_block % 8 != 0 || (reinterpret_cast<uintptr_t>(x) & (x_dtype == kF32 ? 31 : 15)) != 0 ||
+      (reinterpret_cast<uintptr_t>(w) & 15) != 0)
+    return kBadArgument;
+  const dim3 grid((rows + 127) / 128, blocks, (outer + 63) / 64);
+  if (grid.z > 65535) return kBadArgument;
+  hipStream_t s = (hipStream_t)stream;
+#define TLIE_CASE(XC, X, YC, Y)                                                                                   \
+  if (x_dtype == XC && y_dtype == YC) {                                                                           \
+    hipLaunchKernelGGL((block_linear_mfma_kernel<X, Y>), grid, dim3(256), 0, s, (const X*)x, x_row, x_block,        \
+                       (const bf16*)w, (const bf16*)bias, (Y*)y, y_row, y_block, rows, inner, outer);             \
+    return launch_status();                                                                                       \
+  }
+  TLIE_CASE(kBF16, bf16, kBF16, bf16)
+  TLIE_CASE(kBF16, bf16, kF32, float)
+  TLIE_CASE(kF32, float, kF32, float)
+  TLIE_CASE(kF32, float, kBF16, bf16)
+#undef TLIE_CASE
+  return kBadArgument;
+}
 
 // x: rows of x_row elements, block b's `inner` values from b * x_block on; wt: [blocks][inner][outer];
 // bias: [blocks][outer] or null; y: rows of y_row elements, block b's `outer` results from b * y_block on.

@@ -48,7 +48,7 @@ struct Plan {
 Api api;
 std::mutex guard;
 std::map<int, hipblasLtHandle_t> handles;                              // by device
-std::map<std::tuple<int, int, int, int, int, size_t>, Plan> plans;    // by (device, M, N, K, type of y, workspace)
+std::map<std::tuple<int, int, int, int, int, size_t>, Plan> plans;    // by (device, M, N, K, type of y and whether a bias joins, workspace)
 #endif
 
 }  // namespace
@@ -84,9 +84,10 @@ extern "C" int tlie_library_gemm_init(const char* path) {
 
 // x [M, K], w [N, K]: bfloat16; y [M, N]: bfloat16, or float when y_float != 0 (the sums are float either way);
 // row-major, dense.  workspace: device memory the library may use.
+// bias (or null): bfloat16 [N], added to the float sums in the library's own epilogue, before the result is rounded.
 // Returns 0, or -3 when the library has no algorithm for the shape (or is not there): nothing was launched then.
-extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int y_float, int M, int N, int K, void* workspace,
-                                 size_t workspace_bytes, void* stream) {
+static int library_gemm(const void* x, const void* w, const void* bias, void* y, int y_float, int M, int N, int K, void* workspace,
+                        size_t workspace_bytes, void* stream) {
 #ifdef TLIE_HAVE_HIPBLASLT
   if (M <= 0 || N <= 0 || K <= 0) return tlie::kBadArgument;
   if (!api.ready) return kUnavailable;
@@ -99,7 +100,7 @@ extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int y_fl
     if (api.create(&made) != HIPBLAS_STATUS_SUCCESS) return kUnavailable;
     handle = handles.emplace(device, made).first;
   }
-  const auto key = std::make_tuple(device, M, N, K, y_float != 0 ? 1 : 0, workspace_bytes);
+  const auto key = std::make_tuple(device, M, N, K, (y_float != 0 ? 1 : 0) + (bias != nullptr ? 2 : 0), workspace_bytes);
   auto found = plans.find(key);
   if (found == plans.end()) {
     // In the library's column-major terms: y^T [N x M] = op_T(W as K x N) . (x as K x M)
@@ -113,6 +114,14 @@ extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int y_fl
                 api.layout_create(&plan.x, HIP_R_16BF, K, M, K) == HIPBLAS_STATUS_SUCCESS &&
                 api.layout_create(&plan.y, y_float != 0 ? HIP_R_32F : HIP_R_16BF, N, M, N) == HIPBLAS_STATUS_SUCCESS &&
                 api.preference_create(&preference) == HIPBLAS_STATUS_SUCCESS &&
+                (bias == nullptr || [&] {
+                  // (the result's rows, in the library's column-major terms, are the outputs: the bias has one entry a row)
+                  const hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
+                  const hipDataType bias_type = HIP_R_16BF;
+                  return api.desc_set(plan.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue)) == HIPBLAS_STATUS_SUCCESS &&
+                         api.desc_set(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)) == HIPBLAS_STATUS_SUCCESS &&
+                         api.desc_set(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)) == HIPBLAS_STATUS_SUCCESS;
+                }()) &&
                 api.preference_set(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &workspace_bytes,
                                    sizeof(workspace_bytes)) == HIPBLAS_STATUS_SUCCESS;
     if (made) {
@@ -135,12 +144,27 @@ extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int y_fl
   }
   const Plan& plan = found->second;
   if (!plan.usable) return kUnavailable;
+  // the plan serves every product of its shape: the bias of this one goes into its description now (the launch reads it)
+  if (bias != nullptr && api.desc_set(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias)) != HIPBLAS_STATUS_SUCCESS)
+    return kUnavailable;
   const float one = 1.f, zero = 0.f;
   const hipblasStatus_t status = api.matmul(handle->second, plan.desc, &one, w, plan.w, x, plan.x, &zero, y, plan.y, y, plan.y,
                                             &plan.algo, workspace, workspace_bytes, (hipStream_t)stream);
   return status == HIPBLAS_STATUS_SUCCESS ? tlie::kOk : tlie::kLaunchFailed;
 #else
-  (void)x, (void)w, (void)y, (void)y_float, (void)M, (void)N, (void)K, (void)workspace, (void)workspace_bytes, (void)stream;
+  (void)x, (void)w, (void)bias, (void)y, (void)y_float, (void)M, (void)N, (void)K, (void)workspace, (void)workspace_bytes, (void)stream;
   return kUnavailable;
 #endif
+}
+
+extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int y_float, int M, int N, int K, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  return library_gemm(x, w, nullptr, y, y_float, M, N, K, workspace, workspace_bytes, stream);
+}
+
+// The same with a bias [N] (bfloat16) that joins the float sums inside the library's kernel.
+extern "C" int tlie_library_gemm_bias(const void* x, const void* w, const void* bias, void* y, int y_float, int M, int N, int K,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  if (bias == nullptr) return tlie::kBadArgument;
+  return library_gemm(x, w, bias, y, y_float, M, N, K, workspace, workspace_bytes, stream);
 }

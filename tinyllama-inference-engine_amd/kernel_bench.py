@@ -279,7 +279,8 @@ def bench_design_kernels(sizes: dict, batch: int = 8, context: int = 2048, promp
             read_bytes=tokens * (fused.cols * 2 + lh * (ldim + lrot) * 2 + (key + rank) * 2))
         q_plain, q_wide = launch(0)
         up_keys, up_values = rand(lh, ldim, rank), rand(lh, rank, lv)
-        launch = lambda i: ops.block_linear(q_plain, 0, lh * ldim, ldim, up_keys, None, q_wide, 0, lh * key, key, tokens)
+        up_keys_rows, up_values_rows = up_keys.transpose(1, 2).contiguous(), up_values.transpose(1, 2).contiguous()
+        launch = lambda i: ops.block_linear(q_plain, 0, lh * ldim, ldim, up_keys, None, q_wide, 0, lh * key, key, tokens, weight=up_keys_rows)
         row(f"{label}: heads' queries onto the latent space [{lh} x {ldim} x {rank}]", _timed(launch, 4, samples),
             **({"read_bytes": lh * ldim * rank * 2 + tokens * lh * (ldim + rank) * 2} if decode else {"flops": 2.0 * tokens * lh * ldim * rank}))
         latent_sink = rand(lh, scale=1.0, dtype=f32)
@@ -294,7 +295,7 @@ def bench_design_kernels(sizes: dict, batch: int = 8, context: int = 2048, promp
                 flops=2.0 * lh * (key + rank) * tokens * (tokens + 1) / 2)
         attended = rand(tokens, lh * key, scale=1.0)
         values = torch.empty((tokens, lh * lv), dtype=bf, device=device)
-        launch = lambda i: ops.block_linear(attended, 0, lh * key, key, up_values, None, values, 0, lh * lv, lv, tokens)
+        launch = lambda i: ops.block_linear(attended, 0, lh * key, key, up_values, None, values, 0, lh * lv, lv, tokens, weight=up_values_rows)
         row(f"{label}: attended latent vectors onto the heads' values [{lh} x {rank} x {lv}]", _timed(launch, 4, samples),
             **({"read_bytes": lh * rank * lv * 2 + tokens * lh * (rank + lv) * 2} if decode else {"flops": 2.0 * tokens * lh * rank * lv}))
         # ---- the recurrence: convolution, gates, scan -------------------------------------------------------------
@@ -307,7 +308,8 @@ def bench_design_kernels(sizes: dict, batch: int = 8, context: int = 2048, promp
         u = launch(0)
         gates_t, gate_bias = rand(lru_blocks, inside, 2 * inside), rand(lru_blocks, 2 * inside)
         gates = torch.empty((tokens, 2 * lru), dtype=f32, device=device)
-        launch = lambda i: ops.block_linear(u, 0, lru, inside, gates_t, gate_bias, gates, 0, 2 * lru, 2 * inside, tokens)
+        gates_rows = gates_t.transpose(1, 2).contiguous()
+        launch = lambda i: ops.block_linear(u, 0, lru, inside, gates_t, gate_bias, gates, 0, 2 * lru, 2 * inside, tokens, weight=gates_rows)
         row(f"{label}: the recurrence's gates [{lru_blocks} x {inside} x {2 * inside}]", _timed(launch, 4, samples),
             **({"read_bytes": lru_blocks * inside * 2 * inside * 2 + tokens * lru * 12} if decode else {"flops": 4.0 * tokens * lru * inside}))
         lam = rand(lru, scale=1.0)

@@ -388,12 +388,19 @@ def qkv_place(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor | No
     return q_out
 
 
+BLOCK_LINEAR_MANY_ROWS = 16    # rows beyond which the block-diagonal product goes to the matrix cores (where it can)
+
+
 def block_linear(x: torch.Tensor, x_offset: int, x_row: int, x_block: int, weight_t: torch.Tensor, bias: torch.Tensor | None,
-                 out: torch.Tensor, out_offset: int, out_row: int, out_block: int, rows: int) -> None:
+                 out: torch.Tensor, out_offset: int, out_row: int, out_block: int, rows: int,
+                 weight: torch.Tensor | None = None) -> None:
     """Block-diagonal product: for each of weight_t's blocks b, rows of `inner` values that lie in the flat
     array x at x_offset + row * x_row + b * x_block are multiplied by weight_t[b] ([inner, outer], the
     block's matrix transposed) and, plus bias[b], written to the flat array `out` at out_offset + row *
-    out_row + b * out_block.  Sums are float."""
+    out_row + b * out_block.  Sums are float.
+    weight: the same matrices as they are stored, [blocks, outer, inner], in bfloat16: with it a step of more than
+    BLOCK_LINEAR_MANY_ROWS rows goes to the matrix cores (x, if float, is rounded to bfloat16 as an operand), when
+    inner is a multiple of 32 and x's offset and strides are multiples of 8."""
     _device_tensor(x, "x", (torch.float32, torch.bfloat16))
     _device_tensor(weight_t, "weight", (torch.float32, torch.bfloat16))
     _device_tensor(out, "out", (torch.float32, torch.bfloat16))
@@ -414,6 +421,18 @@ def block_linear(x: torch.Tensor, x_offset: int, x_row: int, x_block: int, weigh
         raise invalid_shape("block_linear: the strides reach beyond out")
     x_address = x.data_ptr() + x_offset * x.element_size()
     out_address = out.data_ptr() + out_offset * out.element_size()
+    if (weight is not None and rows > BLOCK_LINEAR_MANY_ROWS and weight.dtype == torch.bfloat16 and inner % 32 == 0
+            and x_offset % 8 == 0 and x_row % 8 == 0 and x_block % 8 == 0 and x_address % 32 == 0):
+        _device_tensor(weight, "weight (as stored)", torch.bfloat16)
+        if weight.shape != (blocks, outer, inner):
+            raise invalid_shape("block_linear: the stored weight must be [blocks, outer, inner]")
+        if bias is not None and bias.dtype != torch.bfloat16:
+            raise EngineError(ErrorCode.INVALID_DTYPE, "block_linear: on the matrix cores the bias is bfloat16")
+        _check(library().tlie_block_linear_mfma(ctypes.c_void_p(x_address), dtype_code(x.dtype), ctypes.c_longlong(x_row),
+                                                ctypes.c_longlong(x_block), _ptr(weight), _ptr(bias), ctypes.c_void_p(out_address),
+                                                dtype_code(out.dtype), ctypes.c_longlong(out_row), ctypes.c_longlong(out_block),
+                                                rows, blocks, inner, outer, _stream()), "block_linear_mfma")
+        return
     _check(library().tlie_block_linear(ctypes.c_void_p(x_address), dtype_code(x.dtype), ctypes.c_longlong(x_row),
                                        ctypes.c_longlong(x_block), _ptr(weight_t), dtype_code(weight_t.dtype), _ptr(bias),
                                        ctypes.c_void_p(out_address), dtype_code(out.dtype), ctypes.c_longlong(out_row),
@@ -551,17 +570,20 @@ def gemm_generic(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | Non
 
 
 # state: None (not tried), True, False (not there); fallbacks: products that took this library's plain kernel instead
-_library_gemm = {"state": None, "workspace": {}, "fallbacks": 0, "warned": set()}
+_library_gemm = {"state": None, "workspace": {}, "fallbacks": 0, "warned": set(), "no_bias_epilogue": set()}
 LIBRARY_WORKSPACE_BYTES = 32 << 20
 
 
-def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+               bias: torch.Tensor | None = None) -> torch.Tensor:
     """y = x . W^T of bfloat16 operands through the vendor's library (hipBLASLt), for steps of many
     rows; y in bfloat16, or in float32 (the output head's logits).  The library is called
     directly, with its plan for the shape kept (half the host time of torch.mm, which a step of
     prompt portions calls four times a layer); where that is not possible (the library's file
     is not beside torch, or it has no algorithm for the shape) this library's plain kernel makes the
-    product."""
+    product.  bias (bfloat16, one entry per row of W): joins the float sums in the library's own kernel; where
+    the library offers nothing for that, the product is made without it and a kernel of this library adds it to
+    the float result (either way the sum is rounded once)."""
     if out_dtype not in (torch.bfloat16, torch.float32):
         raise EngineError(ErrorCode.INVALID_DTYPE, f"library_mm gives bfloat16 or float32, not {out_dtype}")
     _device_tensor(x, "x", torch.bfloat16)
@@ -574,6 +596,29 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = t
         path = os.path.join(os.path.dirname(torch.__file__), "lib", "libhipblaslt.so")
         torch.mm(x[:1], weight[:1].t())                       # torch loads and sets up its copy of the library first
         state["state"] = os.path.isfile(path) and library().tlie_library_gemm_init(path.encode()) == 0
+    if bias is not None:
+        _device_tensor(bias, "bias", torch.bfloat16)
+        if bias.shape != (weight.shape[0],):
+            raise invalid_shape("library_mm: the bias needs one entry per row of W")
+        if state["state"] and x.dim() == 2 and x.shape[0] > 0 and (tuple(x.shape), tuple(weight.shape)) not in state["no_bias_epilogue"]:
+            _device_tensor(x, "x", torch.bfloat16)
+            _device_tensor(weight, "weight", torch.bfloat16)
+            if weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+                raise invalid_shape(f"library_mm: x {list(x.shape)} and weight {list(weight.shape)} do not fit")
+            index = x.device.index or 0
+            if index not in state["workspace"]:
+                state["workspace"][index] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
+            workspace = state["workspace"][index]
+            out = torch.empty((x.shape[0], weight.shape[0]), dtype=out_dtype, device=x.device)
+            status = library().tlie_library_gemm_bias(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), int(out_dtype == torch.float32),
+                                                      x.shape[0], weight.shape[0], x.shape[1], _ptr(workspace),
+                                                      ctypes.c_size_t(workspace.numel()), _stream())
+            if status == 0:
+                return out
+            if status != -3:
+                _check(status, "library_gemm_bias")
+            state["no_bias_epilogue"].add((tuple(x.shape), tuple(weight.shape)))       # (not asked for again)
+        return add_bias(library_mm(x, weight, torch.float32), bias, out_dtype)
     if state["state"] and x.shape[0] > 0:
         index = x.device.index or 0
         if index not in state["workspace"]:

@@ -71,6 +71,7 @@ class LatentAttention(Mixer):
             self.inv_freq = table[0]
         self.names = {**self.NAMES, **dict(spec.get("names") or {})}
         self.first = self.o = self.down_norm = self.up_keys = self.up_values_t = self.sink = None
+        self.up_keys_rows = self.up_values_rows = None
 
     @classmethod
     def tensor_specs(cls, spec, prefix):
@@ -97,6 +98,11 @@ class LatentAttention(Mixer):
         # vector to its values through W_uv ([value_dim, rank] per head: transposed here)
         self.up_keys = keep(weights[prefix + names["up_keys"]].reshape(self.heads, self.plain, self.rank).contiguous())
         self.up_values_t = keep(weights[prefix + names["up_values"]].reshape(self.heads, self.dv, self.rank).transpose(1, 2).contiguous())
+        # and as the product on the matrix cores wants them (steps of many rows, bfloat16), [outer, inner]
+        self.up_keys_rows = self.up_values_rows = None
+        if self.dtype == torch.bfloat16 and self.up_keys.dtype == torch.bfloat16:
+            self.up_keys_rows = keep(self.up_keys.transpose(1, 2).contiguous())
+            self.up_values_rows = keep(weights[prefix + names["up_values"]].reshape(self.heads, self.dv, self.rank).contiguous())
         self.o = Linear(weights[prefix + names["o"]], None, self.dtype, keep=keep)
         if self.has_sink:
             self.sink = keep(weights[prefix + names["sink"]].float().contiguous())
@@ -117,7 +123,7 @@ class LatentAttention(Mixer):
                                            self.down_norm, self.norm_eps, binding.cache, self.heads, self.plain, self.rot,
                                            self.rank, self.dtype, wide_values=self.wide_values)
         ops.block_linear(q_plain, 0, self.heads * self.plain, self.plain, self.up_keys, None,
-                         q_wide, 0, self.heads * key, key, tokens)
+                         q_wide, 0, self.heads * key, key, tokens, weight=self.up_keys_rows)
         value_dim = key if self.wide_values else self.rank
         if self.wide_values and ops.attention_mfma_takes(self.dtype, key, binding.cache.shape[-1] // key):
             tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, self.heads, 1, key)
@@ -130,5 +136,5 @@ class LatentAttention(Mixer):
         # (of every head's attended vector the first rank dims: with wide values the rest are zeros)
         values = torch.empty((tokens, self.heads * self.dv), dtype=self.dtype, device=attended.device)
         ops.block_linear(attended, 0, self.heads * value_dim, value_dim, self.up_values_t, None,
-                         values, 0, self.heads * self.dv, self.dv, tokens)
+                         values, 0, self.heads * self.dv, self.dv, tokens, weight=self.up_values_rows)
         return self.o(values)

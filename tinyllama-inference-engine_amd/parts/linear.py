@@ -72,8 +72,8 @@ class Linear:
             if x.dim() != 2 or x.shape[1] != self.in_features:
                 raise ops.invalid_shape(f"linear: x {list(x.shape)} does not fit weight {list(self.weight.shape)}")
             if self.bias is not None:
-                # the library's product comes without the bias: it joins the float32 sums in a kernel of this
-                # library's own, as in the kernels that add it themselves, and the sum is rounded once
-                return Product(ops.add_bias(ops.library_mm(x, self.weight, torch.float32), self.bias, out_dtype), 1)
+                # the bias joins the float32 sums, as in the kernels that add it themselves, and the sum is rounded
+                # once: in the library's own kernel, or where it offers none for that in a kernel of this library
+                return Product(ops.library_mm(x, self.weight, out_dtype, bias=self.bias), 1)
             return Product(ops.library_mm(x, self.weight, out_dtype), 1)   # (float32: the output head's logits for many rows)
         return ops.gemm_generic(x, self.weight, self.bias, out_dtype)

@@ -9,8 +9,9 @@ Per token, from the mixer's input h, with `width` channels:
     out = W_o (S * y)
 What a request carries from token to token is S and the convolution's last taps - 1 inputs: a row of
 [taps, width] floats in the cache manager's state area, zeroed when the request is admitted.  The two
-projections are one product; the convolution, the gates (from the float u, with float sums), the decay
-and the state are float whatever the activation type.
+projections are one product; the convolution, the gates' sigmoids, the decay and the state are float whatever
+the activation type.  The gates' products have float sums; in a bfloat16 step of many rows they run on the matrix
+cores, whose operands are bfloat16 (u is rounded as it becomes one; the u that drives the state stays float).
 """
 from __future__ import annotations
 
@@ -53,7 +54,7 @@ class GatedRecurrence(Mixer):
             raise invalid_config("gated_recurrence: width must be a positive multiple of blocks, taps positive")
         self.block_width = self.width // self.blocks
         self.names = {**self.NAMES, **dict(spec.get("names") or {})}
-        self.first = self.o = self.conv = self.conv_bias = self.gates_t = self.gate_bias = self.lam = None
+        self.first = self.o = self.conv = self.conv_bias = self.gates_t = self.gate_bias = self.lam = self.gates_rows = None
 
     @classmethod
     def tensor_specs(cls, spec, prefix):
@@ -79,6 +80,10 @@ class GatedRecurrence(Mixer):
         # both gates of a block as one matrix [inner, 2 * inside]: r's outputs, then i's (stored [out, in] per block)
         self.gates_t = keep(torch.cat([get("recurrence_gate").transpose(1, 2), get("input_gate").transpose(1, 2)], dim=2).contiguous())
         self.gate_bias = keep(torch.cat([get("recurrence_gate_bias"), get("input_gate_bias")], dim=1).contiguous())
+        # and as the product on the matrix cores wants them (steps of many rows, bfloat16): [2 * inside, inner] a block
+        self.gates_rows = None
+        if self.dtype == torch.bfloat16 and self.gates_t.dtype == torch.bfloat16:
+            self.gates_rows = keep(torch.cat([get("recurrence_gate"), get("input_gate")], dim=1).contiguous())
         self.lam = keep(get("decay").contiguous())
         self.o = Linear(get("o"), None, self.dtype, keep=keep)
 
@@ -92,7 +97,7 @@ class GatedRecurrence(Mixer):
         u = ops.causal_conv(fused, width, self.conv, self.conv_bias, binding.state, ctx.token_seq, ctx.token_slot, ctx.seq_start)
         gates = torch.empty((tokens, 2 * width), dtype=torch.float32, device=u.device)
         ops.block_linear(u, 0, width, self.block_width, self.gates_t, self.gate_bias,
-                         gates, 0, 2 * width, 2 * self.block_width, tokens)
+                         gates, 0, 2 * width, 2 * self.block_width, tokens, weight=self.gates_rows)
         mixed = ops.gated_recurrence(fused, width, 0, u, gates, self.lam, self.decay, binding.state, ctx.seq_start, ctx.seq_slot,
                                      self.block_width, self.dtype, max_new=ctx.max_new)
         return self.o(mixed)
