@@ -118,6 +118,19 @@ __device__ __forceinline__ float sum_splits(const D* __restrict__ first, int nsp
   return (a + b) + (c + d);
 }
 
+// The gate of a gated feed-forward, from a gate g and an up u (both float).
+// kind 0: silu(g) * u (reference: (g / (1 + exp(-g))) * u in float, src/cuda/kernels.cu:198-206).
+// kind 1: g and u clamped first, g from above only (g = min(g, limit), u in [-limit, limit]), then
+//         g * sigmoid(alpha * g) * (u + 1).
+__device__ __forceinline__ float gated_value(float g, float u, int kind, float alpha, float limit) {
+  if (kind == 0) return (g / (1.f + expf(-g))) * u;
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return (g / (1.f + expf(-alpha * g))) * (u + 1.f);
+}
+
+constexpr int kGateSilu = 0, kGateClampedSwish = 1;
+
 // Error codes returned by the C entry points (0 = launched).
 constexpr int kOk = 0;
 constexpr int kBadArgument = -1;   // a size or dtype the kernel does not take

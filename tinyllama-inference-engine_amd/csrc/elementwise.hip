@@ -98,17 +98,6 @@ __global__ void add_rmsnorm_wide_kernel(float* __restrict__ residual, const D* _
   }
 }
 
-// ---- the gate of a gated feed-forward, from a gate g and an up u (both float) -------------------------
-// kind 0: silu(g) * u (reference: (g / (1 + exp(-g))) * u in float, src/cuda/kernels.cu:198-206).
-// kind 1: g and u clamped first, g from above only (g = min(g, limit), u in [-limit, limit]), then
-//         g * sigmoid(alpha * g) * (u + 1).
-__device__ __forceinline__ float gated_value(float g, float u, int kind, float alpha, float limit) {
-  if (kind == 0) return (g / (1.f + expf(-g))) * u;
-  g = fminf(g, limit);
-  u = fminf(fmaxf(u, -limit), limit);
-  return (g / (1.f + expf(-alpha * g))) * (u + 1.f);
-}
-
 // ---- act[t, i] = silu(gate[t, i]) * up[t, i]; gate_up is [rows, 2 * inter], either [gate | up] or,
 // interleaved, g0 u0 g1 u1 ... (the layout the gated product of few rows wants of its weight) -------
 // reference: (g / (1 + exp(-g))) * u in float (src/cuda/kernels.cu:198-206)
@@ -202,6 +191,60 @@ __global__ void norm_add_rmsnorm_kernel(float* __restrict__ residual, const D* _
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_float<O>(row_cache[i] * scale * to_float(weight[i]));
 }
 
+// The same with eight elements a thread (16-byte loads and stores): hidden % 8 == 0; the summands of a split
+// product are added in the order of their index.
+template <typename D, typename W, typename O>
+__global__ void norm_add_rmsnorm_wide_kernel(float* __restrict__ residual, const D* __restrict__ delta, int nsplit,
+                                             size_t split_stride, const W* __restrict__ post_weight, float post_eps,
+                                             const W* __restrict__ weight, float eps, O* __restrict__ out,
+                                             const int* __restrict__ rows, int hidden) {
+  extern __shared__ float row_cache[];           // hidden floats, then 16 for the reductions
+  float* scratch = row_cache + hidden;
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float* res = residual + static_cast<size_t>(src) * hidden;
+  float square = 0.f;
+  for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) {
+    const D* part = delta + static_cast<size_t>(src) * hidden + i;
+    float d[8];
+    load8(part, d);
+    for (int s = 1; s < nsplit; ++s) {
+      float more[8];
+      load8(part + s * split_stride, more);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) d[j] += more[j];
+    }
+    store8(row_cache + i, d);                    // (a thread reads back only what it wrote itself)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) square += d[j] * d[j];
+  }
+  const float post_scale = rsqrtf(block_sum(square, scratch) / static_cast<float>(hidden) + post_eps);
+  square = 0.f;
+  for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) {
+    float v[8], d[8], w[8];
+    load8(res + i, v);
+    load8(row_cache + i, d);
+    load8(post_weight + i, w);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = v[j] + d[j] * post_scale * w[j];
+    if (!rows) store8(res + i, v);
+    store8(row_cache + i, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) square += v[j] * v[j];
+  }
+  if (out == nullptr) return;                    // (the same for the whole grid)
+  const float scale = rsqrtf(block_sum(square, scratch) / static_cast<float>(hidden) + eps);
+  O* o = out + static_cast<size_t>(r) * hidden;
+  for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) {
+    float v[8], w[8];
+    load8(row_cache + i, v);
+    load8(weight + i, w);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = v[j] * scale * w[j];
+    store8(o + i, v);
+  }
+}
+
 // ---- out[r, c] = product[r, c] + bias[c] ------------------------------------------------------
 // For a product that a library made without its bias (steps of many rows): the bias joins the
 // float sums, as in the kernels that add it themselves, and the result is rounded once.
@@ -286,8 +329,20 @@ extern "C" int tlie_norm_add_rmsnorm(float* residual, const void* delta, int del
   if (lds > 160 * 1024) return kBadArgument;
   const int threads = hidden >= 4096 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 256 : 64));
   hipStream_t s = (hipStream_t)stream;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(residual) | reinterpret_cast<uintptr_t>(delta) | reinterpret_cast<uintptr_t>(post_weight) |
+                         reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out)) & 31) == 0;
+  const size_t delta_size = delta_dtype == kF32 ? 4 : 2;
+  const bool wide = (hidden & 7) == 0 && aligned && (nsplit == 1 || (static_cast<size_t>(split_stride) * delta_size) % 32 == 0);
+  const int chunks = hidden / 8;
+  const int wide_threads = chunks >= 1024 ? 1024 : (chunks + 63) / 64 * 64;
 #define TLIE_CASE(DC, D, WC, W, OC, O)                                                                              \
   if (delta_dtype == DC && weight_dtype == WC && out_dtype == OC) {                                                 \
+    if (wide) {                                                                                                     \
+      hipLaunchKernelGGL((norm_add_rmsnorm_wide_kernel<D, W, O>), dim3(num_rows), dim3(wide_threads), lds, s, residual, \
+                         (const D*)delta, nsplit, (size_t)split_stride, (const W*)post_weight, post_eps,            \
+                         (const W*)weight, eps, (O*)out, rows, hidden);                                              \
+      return launch_status();                                                                                       \
+    }                                                                                                               \
     hipLaunchKernelGGL((norm_add_rmsnorm_kernel<D, W, O>), dim3(num_rows), dim3(threads), lds, s, residual,          \
                        (const D*)delta, nsplit, (size_t)split_stride, (const W*)post_weight, post_eps,              \
                        (const W*)weight, eps, (O*)out, rows, hidden);                                                \

@@ -58,6 +58,8 @@ struct RowsArgs {
   // outputs
   float* y;                   // store: [M, N]
   uint16_t* act;              // SiLU: [M, N / 2]
+  int gate_kind;              // which gate the gated epilogue applies (see gated_value), with its constants
+  float gate_alpha, gate_limit;
   float* residual;            // residual: [M, N], updated in place
   const uint16_t* next_weight;  // residual: [N] bfloat16 weight of the next norm, or null
   const float* next_weight_f32; // the same when that weight is kept in float32
@@ -270,7 +272,7 @@ gemm_rows_kernel(const RowsArgs a) {
       } else if (EPILOGUE == kEpilogueSilu) {
         const float up = __shfl_down(value, 1, 64);          // the odd row next to this even one
         if (live && (nn & 1) == 0) {
-          const float gated = (value / (1.f + expf(-value))) * up;
+          const float gated = gated_value(value, up, a.gate_kind, a.gate_alpha, a.gate_limit);
           a.act[static_cast<size_t>(token) * (a.N / 2) + (n >> 1)] = __bfloat16_as_ushort(__float2bfloat16(gated));
         }
       } else if (EPILOGUE == kEpilogueRope) {
@@ -395,7 +397,8 @@ extern "C" int tlie_gemm_rows(const void* x, const void* w, const void* bias, in
                               const void* next_weight, int next_weight_dtype, void* xg, float* ssq_out,
                               const int* positions, const int* slot_map, const float* inv_freq, int rot_dim, int nq,
                               int nkv, int d, int page_size, void* q_out, void* cache, int waves, int rows_per_block,
-                              void* stream) {
+                              int gate_kind, float gate_alpha, float gate_limit, void* stream) {
+  if (gate_kind != kGateSilu && gate_kind != kGateClampedSwish) return kBadArgument;
   if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K & 7) != 0 || (waves != 2 && waves != 4 && waves != 8 && waves != 16)) return kBadArgument;
   if (!(rows_per_block >= 2 && rows_per_block <= 16 && rows_per_block % 2 == 0) && !(rows_per_block == 32 && waves <= 8)) return kBadArgument;
   if (ssq_in != nullptr && (strips_in <= 0 || width <= 0)) return kBadArgument;
@@ -416,6 +419,7 @@ extern "C" int tlie_gemm_rows(const void* x, const void* w, const void* bias, in
   a.next_weight_f32 = next_weight_dtype == kBF16 ? nullptr : (const float*)next_weight;
   a.xg = (uint16_t*)xg, a.ssq_out = ssq_out;
   a.positions = positions, a.slot_map = slot_map, a.inv_freq = inv_freq, a.rot_dim = rot_dim;
+  a.gate_kind = gate_kind, a.gate_alpha = gate_alpha, a.gate_limit = gate_limit;
   a.nq = nq, a.nkv = nkv, a.d = d, a.page_size = page_size, a.q_out = (uint16_t*)q_out, a.cache = (uint16_t*)cache;
   const dim3 grid((N + rows_per_block - 1) / rows_per_block);
   hipStream_t s = (hipStream_t)stream;

@@ -42,7 +42,7 @@ constexpr int kSkinnyPad = 8;                // bf16 elements of padding per LDS
 template <int NT, int RS, int CHUNK, int MINWAVES, int MAXWAVES, bool GATED = false>
 __global__ void __launch_bounds__(64 * MAXWAVES)
 gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias,
-                   float* __restrict__ y, uint16_t* __restrict__ act, int M, int N, int K, int split_len) {
+                   float* __restrict__ y, uint16_t* __restrict__ act, int M, int N, int K, int split_len, int gate_kind, float gate_alpha, float gate_limit) {
   constexpr int kStride = CHUNK + kSkinnyPad;
   constexpr int kSteps = CHUNK / 64;
   __shared__ __attribute__((aligned(16))) uint16_t xs[NT * 16 * kStride];
@@ -156,9 +156,9 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
         const float g0 = acc[r][t][0] + add[0], u0 = acc[r][t][1] + add[1], g1 = acc[r][t][2] + add[2], u1 = acc[r][t][3] + add[3];
         uint16_t* gated = act + static_cast<size_t>(token) * (N / 2) + (n0 >> 1);
         if (n0 + 3 < N)
-          *reinterpret_cast<uint32_t*>(gated) = pack_bf16((g0 / (1.f + expf(-g0))) * u0, (g1 / (1.f + expf(-g1))) * u1);
+          *reinterpret_cast<uint32_t*>(gated) = pack_bf16(gated_value(g0, u0, gate_kind, gate_alpha, gate_limit), gated_value(g1, u1, gate_kind, gate_alpha, gate_limit));
         else if (n0 + 1 < N)
-          gated[0] = __bfloat16_as_ushort(__float2bfloat16((g0 / (1.f + expf(-g0))) * u0));
+          gated[0] = __bfloat16_as_ushort(__float2bfloat16(gated_value(g0, u0, gate_kind, gate_alpha, gate_limit)));
         continue;
       }
       float* out = y + (static_cast<size_t>(split) * M + token) * N + n0;
@@ -182,21 +182,21 @@ namespace {
 
 template <int NT, int RS, bool GATED>
 int launch_skinny(dim3 grid, int waves, hipStream_t s, const uint16_t* x, const uint16_t* w, const uint16_t* bias, float* y,
-                  uint16_t* act, int M, int N, int K, int split_len) {
+                  uint16_t* act, int M, int N, int K, int split_len, int gate_kind, float gate_alpha, float gate_limit) {
   // (the staged chunk is as long as the registers allow for the workgroup's size)
   const dim3 block(64 * waves);
   if (waves == 3) {
     constexpr int kChunk = NT <= 2 ? 512 : 256;
-    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 3, 3, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len);
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 3, 3, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len, gate_kind, gate_alpha, gate_limit);
   } else if (waves <= 4) {
     constexpr int kChunk = NT <= 2 ? 512 : 256;
-    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 4, 4, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len);
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 4, 4, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len, gate_kind, gate_alpha, gate_limit);
   } else if (waves <= 8) {
     constexpr int kChunk = RS == 1 ? 256 : 128;
-    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 5, 8, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len);
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 5, 8, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len, gate_kind, gate_alpha, gate_limit);
   } else {
     if constexpr (RS == 1)
-      hipLaunchKernelGGL((gemm_skinny_kernel<NT, 1, (NT <= 2 ? 256 : 128), 9, 16, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len);
+      hipLaunchKernelGGL((gemm_skinny_kernel<NT, 1, (NT <= 2 ? 256 : 128), 9, 16, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len, gate_kind, gate_alpha, gate_limit);
     else
       return kBadArgument;
   }
@@ -205,11 +205,11 @@ int launch_skinny(dim3 grid, int waves, hipStream_t s, const uint16_t* x, const 
 
 template <bool GATED>
 int dispatch_skinny(dim3 grid, int waves, int strips, int tiles, hipStream_t s, const uint16_t* x, const uint16_t* w,
-                    const uint16_t* bias, float* y, uint16_t* act, int M, int N, int K, int split_len) {
-  if (tiles <= 1) return launch_skinny<1, 1, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len);
-  if (tiles == 2) return launch_skinny<2, 1, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len);
-  if (strips == 1) return launch_skinny<4, 1, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len);
-  return launch_skinny<4, 2, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len);
+                    const uint16_t* bias, float* y, uint16_t* act, int M, int N, int K, int split_len, int gate_kind, float gate_alpha, float gate_limit) {
+  if (tiles <= 1) return launch_skinny<1, 1, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len, gate_kind, gate_alpha, gate_limit);
+  if (tiles == 2) return launch_skinny<2, 1, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len, gate_kind, gate_alpha, gate_limit);
+  if (strips == 1) return launch_skinny<4, 1, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len, gate_kind, gate_alpha, gate_limit);
+  return launch_skinny<4, 2, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len, gate_kind, gate_alpha, gate_limit);
 }
 
 }  // namespace
@@ -220,8 +220,11 @@ int dispatch_skinny(dim3 grid, int waves, int strips, int tiles, hipStream_t s, 
 // than 32 rows of x and up to 8 waves); a workgroup takes 16 * strips * waves rows of W.
 // act (or null): with it, split_len must cover K (one split), N must be even, W's rows alternate gate and up, and
 // bfloat16 silu(gate) * up [M, N / 2] is stored there instead of y (which may then be null).
+// gate_kind, gate_alpha, gate_limit: which gate `act` gets (see gated_value; 0: silu(gate) * up).
 extern "C" int tlie_gemm_skinny(const void* x, const void* w, const void* bias, float* y, void* act, int M, int N, int K,
-                                int split_len, int waves, int strips, void* stream) {
+                                int split_len, int waves, int strips, int gate_kind, float gate_alpha, float gate_limit,
+                                void* stream) {
+  if (gate_kind != kGateSilu && gate_kind != kGateClampedSwish) return kBadArgument;
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) != 0 || split_len <= 0 || (split_len & 63) != 0) return kBadArgument;
   if (waves < 3 || waves > 16 || strips < 1 || strips > 2 || (strips == 2 && (M <= 32 || waves > 8))) return kBadArgument;
   const int nsplit = (K + split_len - 1) / split_len;
@@ -234,6 +237,6 @@ extern "C" int tlie_gemm_skinny(const void* x, const void* w, const void* bias, 
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
-  if (act != nullptr) return dispatch_skinny<true>(grid, waves, strips, tiles, s, xp, wp, bp, y, (uint16_t*)act, M, N, K, split_len);
-  return dispatch_skinny<false>(grid, waves, strips, tiles, s, xp, wp, bp, y, nullptr, M, N, K, split_len);
+  if (act != nullptr) return dispatch_skinny<true>(grid, waves, strips, tiles, s, xp, wp, bp, y, (uint16_t*)act, M, N, K, split_len, gate_kind, gate_alpha, gate_limit);
+  return dispatch_skinny<false>(grid, waves, strips, tiles, s, xp, wp, bp, y, nullptr, M, N, K, split_len, gate_kind, gate_alpha, gate_limit);
 }

@@ -829,12 +829,23 @@ def skinny_gated_plan(rows: int, out_features: int, in_features: int, compute_un
     return best[1], best[2]
 
 
+def _gate_args(gate) -> tuple:
+    """(kind, alpha, limit) as the kernels take them, from None (the SiLU gate) or (name, alpha, limit)."""
+    if gate is None:
+        return 0, ctypes.c_float(1.0), ctypes.c_float(0.0)
+    name, alpha, limit = gate
+    if name not in GATES or (name == "clamped_swish" and not limit > 0.0):
+        raise invalid_argument(f"unknown gate {gate!r}")
+    return GATES[name], ctypes.c_float(alpha), ctypes.c_float(limit)
+
+
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, split_len: int | None = None,
-                waves: int | None = None, strips: int | None = None, gated: bool = False):
+                waves: int | None = None, strips: int | None = None, gated: bool = False, gate=None):
     """y = x . W^T (+ bias) for at most 64 rows of bfloat16 x: float partial sums [nsplit, M, N].
     split_len, waves, strips: the launch shape (see `skinny_plan`, which chooses it when they are not given).
     gated: W's rows alternate gate and up; K is not split, and the kernel stores bfloat16
-    silu(gate) * up [M, N / 2], which is returned as a tensor (no partial sums, no activation kernel)."""
+    silu(gate) * up [M, N / 2], which is returned as a tensor (no partial sums, no activation kernel).
+    gate: (name, alpha, limit) of another gate than SiLU (see `silu_mul`)."""
     _device_tensor(x, "x", torch.bfloat16)
     _device_tensor(weight, "weight", torch.bfloat16)
     if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
@@ -866,11 +877,11 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None
     if gated:
         act = torch.empty((rows, out_features // 2), dtype=torch.bfloat16, device=x.device)
         _check(library().tlie_gemm_skinny(_ptr(x), _ptr(weight), _ptr(bias), _ptr(None), _ptr(act), rows, out_features, in_features,
-                                          split_len, waves, strips, _stream()), "gemm_skinny")
+                                          split_len, waves, strips, *_gate_args(gate), _stream()), "gemm_skinny")
         return act
     out = torch.empty((nsplit, rows, out_features), dtype=torch.float32, device=x.device)
     _check(library().tlie_gemm_skinny(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _ptr(None), rows, out_features, in_features,
-                                      split_len, waves, strips, _stream()), "gemm_skinny")
+                                      split_len, waves, strips, *_gate_args(None), _stream()), "gemm_skinny")
     return Product(out, nsplit)
 
 
@@ -1149,11 +1160,11 @@ class RopeTarget:
 
 def gemm_rows(x, weight: torch.Tensor, bias: torch.Tensor | None, epilogue: str = "store",
               residual: torch.Tensor | None = None, next_norm: tuple | None = None, waves: int | None = None,
-              rows_per_block: int | None = None, rope: RopeTarget | None = None):
+              rows_per_block: int | None = None, rope: RopeTarget | None = None, gate=None):
     """y = x . W^T (+ bias) for at most 16 rows.  x: bfloat16 [M, K], or `NormedRows` (then the
     result's rows are scaled as the norm would have scaled the input).
     epilogue "store": float32 [M, N] as a `Product`.  "silu": W's rows alternate gate and up;
-    returns bfloat16 silu(gate) * up [M, N / 2].  "residual": residual [M, N] += y in place, returns
+    returns bfloat16 silu(gate) * up [M, N / 2] (gate: (name, alpha, limit) of another gate, see `silu_mul`).  "residual": residual [M, N] += y in place, returns
     a `ResidualUpdated`, with the next norm's inputs when next_norm = (weight [N], eps) is given.
     "rope": W is a fused q/k/v weight with rows in the order of `paired_rows`; q and k are rotated,
     k and v written to the cache (as `rope_cache` does), bfloat16 q [M, nq * d] is returned."""
@@ -1235,7 +1246,7 @@ def gemm_rows(x, weight: torch.Tensor, bias: torch.Tensor | None, epilogue: str 
     _check(library().tlie_gemm_rows(_ptr(data), _ptr(weight), _ptr(bias), rows, out_features, in_features, _ptr(ssq_in),
                                     strips_in, in_features, ctypes.c_float(eps), code, _ptr(y), _ptr(act), _ptr(residual),
                                     _ptr(next_weight), next_code, _ptr(xg), _ptr(ssq_out), *rope_args, waves, rows_per_block,
-                                    _stream()), "gemm_rows")
+                                    *_gate_args(gate if epilogue == "silu" else None), _stream()), "gemm_rows")
     if epilogue == "rope":
         return q_out
     if epilogue == "store":

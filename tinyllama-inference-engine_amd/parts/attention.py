@@ -150,7 +150,14 @@ class Attention(Mixer):
             raise invalid_config("attention: a position encoding that is no rotation table goes with the plain options only")
         inv_freq, rot_dim = table if table is not None else (None, 0)
         writes = binding.writes and not self.reads_other_cache
-        q = ops.qkv_place(ops.as_product(self.qkv(x)), ctx.positions, pages.slot_map if writes else ctx.no_slots, inv_freq,
+        q = None
+        if (table is None and self.dv == self.d and self.d % 2 == 0 and not self.reads_other_cache
+                and self.qkv.takes_rows(x.shape[0])):
+            # a step of few rows, one head size, own keys and values: the product places q and writes the cache itself
+            q = self.qkv(x, rope=ops.RopeTarget(ctx.positions, pages.slot_map if writes else ctx.no_slots, None, 0, binding.cache,
+                                                self.nq, self.nkv, self.d))
+        if q is None or isinstance(q, ops.Product):
+            q = ops.qkv_place(ops.as_product(q if q is not None else self.qkv(x)), ctx.positions, pages.slot_map if writes else ctx.no_slots, inv_freq,
                           rot_dim, binding.cache, self.nq, 0 if self.reads_other_cache else self.nkv, self.d, self.dv, self.dtype)
         if self.dv == self.d and ops.attention_mfma_takes(self.dtype, self.d, binding.cache.shape[3] // self.d):
             # bfloat16, one head size: the kernel on the matrix cores (scores, softmax and sink float)

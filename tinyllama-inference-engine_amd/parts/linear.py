@@ -40,14 +40,14 @@ class Linear:
         return ops.gemm_rows_takes(rows, self.weight, self.dtype)
 
     def __call__(self, x, out_dtype: torch.dtype | None = None, whole: bool = False, into=None, gated: bool = False,
-                 rope=None):
+                 rope=None, gate=None):
         """out_dtype: what a dense result is stored in (the skinny kernel's partial sums are float32
         whatever it says).  whole: the caller has no kernel that adds partial sums up, so the
         product must come as one array (the skinny kernel then does not split K).
         into (a `ResidualTarget`): add the result into the residual, if the kernel for this step can
         (then a `ResidualUpdated` comes back, else the result as usual).  gated: the weight's rows
         alternate gate and up; if the kernel for this step can, silu(gate) * up comes back as a
-        tensor, else the product as usual.  rope (an `ops.RopeTarget`; the weight's rows are in
+        tensor, else the product as usual; gate: (name, alpha, limit) of another gate than SiLU.  rope (an `ops.RopeTarget`; the weight's rows are in
         paired order): if the kernel for this step can, q and k are rotated, k and v written to the
         cache and q comes back as a tensor, else the product as usual."""
         out_dtype = out_dtype or self.dtype
@@ -55,7 +55,7 @@ class Linear:
             if into is not None:
                 return ops.gemm_rows(x, self.weight, self.bias, "residual", residual=into.residual, next_norm=into.next_norm)
             if gated:
-                return ops.gemm_rows(x, self.weight, self.bias, "silu")
+                return ops.gemm_rows(x, self.weight, self.bias, "silu", gate=gate)
             if rope is not None:
                 return ops.gemm_rows(x, self.weight, self.bias, "rope", rope=rope)
             if isinstance(x, ops.NormedRows):
@@ -63,7 +63,7 @@ class Linear:
         if isinstance(x, ops.NormedRows):
             raise ops.invalid_argument("this product cannot fold the norm before it; ask takes_rows() first")
         if gated and ops.gemm_skinny_takes(x, self.weight) and self.out_features % 2 == 0:
-            return ops.gemm_skinny(x, self.weight, self.bias, gated=True)     # all of K in a workgroup: the gate is applied there
+            return ops.gemm_skinny(x, self.weight, self.bias, gated=True, gate=gate)     # all of K in a workgroup: the gate is applied there
         if ops.gemm_skinny_takes(x, self.weight) and (not whole or out_dtype == torch.float32):
             split_len = (self.in_features + 63) // 64 * 64 if whole else None
             return ops.gemm_skinny(x, self.weight, self.bias, split_len=split_len)

@@ -71,8 +71,8 @@ class GatedMLP(FeedForward):
         return self.activation == "silu" and self.gate_up.takes_rows(rows)
 
     def forward(self, x, ctx, into=None):
-        # (the products that apply the gate themselves know the SiLU gate only)
-        hidden = self.gate_up(x, gated=self.activation == "silu")
+        gate = None if self.activation == "silu" else (self.activation, self.alpha, self.limit)
+        hidden = self.gate_up(x, gated=True, gate=gate)
         if isinstance(hidden, ops.Product):
             hidden = ops.silu_mul(hidden, self.dtype, interleaved=True, gate=self.activation, alpha=self.alpha, limit=self.limit)
         return self.down(hidden, into=into)
