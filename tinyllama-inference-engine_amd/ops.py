@@ -907,17 +907,22 @@ def attention_tiles(seq_start, groups_per_kv: int, col_tiles: int = 1, seq_len=N
     that the longest are not the last to start.  Returns an int32 array [tiles, 4]:
     (sequence, its first token's index in the step, its number of tokens, the tile's first column)."""
     import numpy as np
-    rows, keys = [], []
-    for seq in range(len(seq_start) - 1):
+    step = 16 * col_tiles
+    parts, keys = [], []
+    for seq in range(len(seq_start) - 1):                  # (a sequence's tiles at once: a prompt has thousands)
         first, count = int(seq_start[seq]), int(seq_start[seq + 1] - seq_start[seq])
-        for col0 in range(0, count * groups_per_kv, 16 * col_tiles):
-            rows.append((seq, first, count, col0))
-            if seq_len is not None:
-                last_token = min(count - 1, (col0 + 16 * col_tiles - 1) // groups_per_kv)
-                keys.append(int(seq_len[seq]) - count + last_token + 1)
-    rows = np.asarray(rows, dtype=np.int32).reshape(-1, 4)
-    if seq_len is not None and len(keys) > 1:
-        rows = rows[np.argsort(-np.asarray(keys), kind="stable")]
+        if count <= 0:
+            continue
+        col0 = np.arange(0, count * groups_per_kv, step, dtype=np.int64)
+        block = np.empty((col0.shape[0], 4), dtype=np.int32)
+        block[:, 0], block[:, 1], block[:, 2], block[:, 3] = seq, first, count, col0
+        parts.append(block)
+        if seq_len is not None:
+            last_token = np.minimum(count - 1, (col0 + step - 1) // groups_per_kv)
+            keys.append(int(seq_len[seq]) - count + last_token + 1)
+    rows = np.concatenate(parts) if parts else np.zeros((0, 4), dtype=np.int32)
+    if seq_len is not None and rows.shape[0] > 1:
+        rows = rows[np.argsort(-np.concatenate(keys), kind="stable")]
     return np.ascontiguousarray(rows)
 
 
