@@ -164,7 +164,7 @@ def _attend(q, k, v, sink, scale, chunk, page_size, cuts, dtype=torch.float32):
 
 
 @pytest.mark.parametrize("heads,groups,d,dv,chunk,page_size", [(4, 2, 16, 24, 24, 16), (3, 3, 9, 5, 7, 4), (2, 1, 72, 8, None, 16),
-                                                               (4, 1, 48, 40, 64, 16), (2, 2, 8, 80, 33, 8)])
+                                                               (4, 1, 56, 40, 60, 16), (2, 2, 8, 80, 33, 8)])
 def test_attention_with_sink_and_chunks(heads, groups, d, dv, chunk, page_size):
     generator = torch.Generator().manual_seed(d * dv)
     tokens = 150
@@ -209,7 +209,7 @@ def _attend_matrix_cores(q, k, v, sink, scale, chunk, page_size, cuts):
 
 
 @pytest.mark.parametrize("heads,groups,d,chunk,page_size,tokens", [(4, 2, 32, 48, 16, 300), (8, 1, 64, 100, 16, 1000), (2, 2, 16, 33, 32, 200),
-                                                                   (6, 3, 128, None, 16, 300), (4, 4, 48, 64, 16, 900)])
+                                                                   (6, 3, 128, None, 16, 300), (4, 4, 80, 72, 16, 900)])
 def test_attention_on_the_matrix_cores_with_sink_and_chunks(heads, groups, d, chunk, page_size, tokens):
     generator = torch.Generator().manual_seed(d + tokens)
     q, k, v = (torch.randn(tokens, n, d, generator=generator).bfloat16().float() for n in (heads, groups, groups))
