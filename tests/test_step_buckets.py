@@ -88,3 +88,32 @@ def test_the_few_rows_products_launch_shape_is_one_the_kernel_takes():
     assert ops.gemm_rows_shape(2560, 2048, "rope", 256, 8) == (16, 10)          # 256 workgroups, one a compute unit
     assert ops.gemm_rows_shape(2048, 2048, "residual", 256, 8) == (16, 16)      # a norm's sums follow: strips of 16
     assert ops.gemm_rows_shape(128256, 4096, "store", 256, 1) == (4, 16) and ops.gemm_rows_shape(128256, 4096, "store", 256, 8) == (4, 32)
+
+
+def test_the_attention_work_list_equals_a_tile_by_tile_walk():
+    """`ops.attention_tiles` makes a sequence's tiles at once; written out tile by tile here, the list must be
+    the same rows in the same order (sequences in order, columns rising, then stably by keys seen, most first)."""
+    import numpy as np
+    from tlie_amd import ops
+
+    def walk(seq_start, per_kv, col_tiles, seq_len):
+        rows, keys = [], []
+        for seq in range(len(seq_start) - 1):
+            first, count = int(seq_start[seq]), int(seq_start[seq + 1] - seq_start[seq])
+            for col0 in range(0, count * per_kv, 16 * col_tiles):
+                rows.append((seq, first, count, col0))
+                keys.append(int(seq_len[seq]) - count + min(count - 1, (col0 + 16 * col_tiles - 1) // per_kv) + 1 if seq_len is not None else 0)
+        rows = np.asarray(rows, dtype=np.int32).reshape(-1, 4)
+        if seq_len is not None and len(keys) > 1:
+            rows = rows[np.argsort(-np.asarray(keys), kind="stable")]
+        return rows
+    rng = np.random.default_rng(3)
+    for _ in range(100):
+        counts = rng.integers(0, 90, rng.integers(1, 7))
+        start = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+        lengths = (counts + rng.integers(0, 400, counts.shape[0])).astype(np.int32)
+        per_kv, col_tiles = int(rng.choice([1, 3, 8, 32])), int(rng.choice([1, 2, 4, 8]))
+        for seq_len in (None, lengths):
+            made = ops.attention_tiles(start, per_kv, col_tiles, seq_len)
+            assert made.dtype == np.int32 and made.flags["C_CONTIGUOUS"]
+            assert np.array_equal(made, walk(start, per_kv, col_tiles, seq_len))
