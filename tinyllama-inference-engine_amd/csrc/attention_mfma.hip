@@ -96,8 +96,11 @@ constexpr int attention_max_waves(int dt, int ct) {
 // longer than what a wave can issue meanwhile), so for head sizes up to 64 the compiler is asked to
 // stay within the registers of 4 waves a SIMD with one column group and 3 with two, where it would
 // take those of 3 and 2 (a prompt of 2048 tokens 53 -> 51 us, of 4096 158 -> 150).
-template <int DT, int CT, bool SHARED>
-__global__ void __launch_bounds__(SHARED ? 512 : 64 * attention_max_waves(DT, CT), (SHARED && DT <= 4) ? (CT == 1 ? 4 : 3) : 1)
+// EXTRA: the kernel also takes chunks of positions and a sink; without it `chunk` and `sink` are not looked
+// at, and the code is the plain causal (or windowed) kernel's, instruction for instruction (the variant that
+// shares keys through LDS is compiled to a tight register budget, which the additions do not fit).
+template <int DT, int CT, bool SHARED, bool EXTRA>
+__global__ void __launch_bounds__(SHARED ? 512 : 64 * attention_max_waves(DT, CT), (SHARED && DT <= 4 && !EXTRA) ? (CT == 1 ? 4 : 3) : 1)
 attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache,
                       const int* __restrict__ block_table, int max_blocks, const int4* __restrict__ tiles,
                       const int* __restrict__ positions, uint16_t* __restrict__ out, float* __restrict__ part_o,
@@ -106,10 +109,10 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   constexpr int D = DT * 16;
   // the first key that the token at position p sees: the window's edge, or the start of the token's own
   // chunk of positions (chunks are counted from position 0), whichever is later; 0 without either
-  const bool bounded = window > 0 || chunk > 0;
+  const bool bounded = window > 0 || (EXTRA && chunk > 0);
   auto lower = [&](int p) {
     int lo = window > 0 ? max(0, p - window + 1) : 0;
-    if (chunk > 0) lo = max(lo, p - p % chunk);
+    if (EXTRA && chunk > 0) lo = max(lo, p - p % chunk);
     return lo;
   };
   constexpr int KS = (DT + 1) / 2;                 // 32-wide k steps of the first product
@@ -563,7 +566,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
     if (!valid_col[ct]) continue;
     if (nsplit == 1) {
       float inv = 1.f / running_sum[ct];
-      if (sink != nullptr) {
+      if (EXTRA && sink != nullptr) {
         // the sink joins the denominator once, as exp(sink): in base 2 and on the common scale of the sums
         const float own = sink[head[ct]] * 1.4426950408889634f;
         const float top = fmaxf(running_max[ct], own);
@@ -681,9 +684,14 @@ static int launch_attention(const void* q, const void* cache, const int* block_t
   // LDS for merging the waves: their maxima and sums, and half as many slots as waves for the results
   const size_t lds = !SHARED && waves > 1 ? (static_cast<size_t>(waves) * CT * 32 + static_cast<size_t>(waves / 2) * CT * DT * 256) * sizeof(float) : 0;
   if (lds > 64 * 1024) return kBadArgument;
-  hipLaunchKernelGGL((attention_mfma_kernel<DT, CT, SHARED>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
-                     (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
-                     part_ml, nsplit, split_len, nq, nkv, page_size, window, chunk, sink, scale_log2, compute_units());
+  if (chunk > 0 || sink != nullptr)
+    hipLaunchKernelGGL((attention_mfma_kernel<DT, CT, SHARED, true>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
+                       (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
+                       part_ml, nsplit, split_len, nq, nkv, page_size, window, chunk, sink, scale_log2, compute_units());
+  else
+    hipLaunchKernelGGL((attention_mfma_kernel<DT, CT, SHARED, false>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
+                       (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
+                       part_ml, nsplit, split_len, nq, nkv, page_size, window, 0, nullptr, scale_log2, compute_units());
   return launch_status();
 }
 

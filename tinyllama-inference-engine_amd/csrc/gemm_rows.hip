@@ -51,15 +51,16 @@ struct RowsArgs {
   const uint16_t* bias;       // [N] or null
   int M, N, K, k_per_wave;    // k_per_wave: multiple of 64
   int rows_per_block;         // even, up to 16; or 32
+  int gate_kind;              // which gate the gated epilogue applies (see gated_value); its constants further down
+                              // (the three lie where the structure had gaps: its size, 192 bytes, is what it was)
   // row scale (null: none)
   const float* ssq_in;        // [strips_in, 16] partial sums of squares of the normed input's rows, over any split of its columns
   int strips_in;
   float inv_width, eps;       // 1 / width of the normed input
+  float gate_alpha;
   // outputs
   float* y;                   // store: [M, N]
   uint16_t* act;              // SiLU: [M, N / 2]
-  int gate_kind;              // which gate the gated epilogue applies (see gated_value), with its constants
-  float gate_alpha, gate_limit;
   float* residual;            // residual: [M, N], updated in place
   const uint16_t* next_weight;  // residual: [N] bfloat16 weight of the next norm, or null
   const float* next_weight_f32; // the same when that weight is kept in float32
@@ -70,9 +71,11 @@ struct RowsArgs {
   const int* slot_map;        // [M] cache row of each token (page * page_size + row), or -1
   const float* inv_freq;      // [rot_dim / 2], or null: no rotation
   int rot_dim, nq, nkv, d, page_size;
+  float gate_limit;
   uint16_t* q_out;            // [M, nq * d]
   uint16_t* cache;            // [pages, 2, nkv, page_size * d]: keys [row][dim], values [dim][row]
 };
+static_assert(sizeof(RowsArgs) == 192, "the arguments of the few-rows product outgrew three cache lines");
 
 // S whole steps of 64 k for every strip: all of W's pieces are asked for first (16 bytes a lane and piece;
 // with 8 steps 16 loads per lane and strip in flight: the weights come from HBM and a wave has nothing
