@@ -932,9 +932,6 @@ def few_rows_route(rows: int, dtype: torch.dtype) -> bool:
     return dtype == torch.bfloat16 and 0 < rows <= ROWS_MAX
 
 
-WIDE_HEAD_KEYS_A_WAVE = 64
-
-
 def attention_plan(ctx, groups_per_kv: int, num_kv_heads: int, head_dim: int):
     """How the tiled attention kernel is launched for the step `ctx` describes: its work list (made
     once per step and group size, kept in `ctx.scratch`; None for a decode step, whose tiles the
@@ -1001,10 +998,8 @@ def attention_plan(ctx, groups_per_kv: int, num_kv_heads: int, head_dim: int):
         # 8 x 2, batch 64 1 x 8)
         nsplit = max(1, min((256 + tiles_all - 1) // tiles_all, 16, (ctx.max_context + 63) // 64))
         waves = 1
-        # (a wave keeps 128 keys or more; of heads wider than 128 dims, where a key is more work, 64)
-        keys_a_wave = 128 if head_dim <= 128 else WIDE_HEAD_KEYS_A_WAVE
         while (waves * 2 <= attention_max_waves(head_dim) and tiles_all * nsplit * waves * 2 <= 2048
-               and ctx.max_context >= nsplit * waves * 2 * keys_a_wave):
+               and ctx.max_context >= nsplit * waves * 2 * 128):
             waves *= 2
         if nsplit > 1 and ctx.max_context <= 256 and attention_max_waves(head_dim) >= 2:
             # up to 256 positions there is nothing to cut: two waves of one workgroup share the keys and the
