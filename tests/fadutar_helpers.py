@@ -46,6 +46,9 @@ CONFIG_Q = {
         {"type": "attention", "mixer": {"heads": 4, "kv_heads": 1, "dim": 9, "vdim": 5, "scale": 0.4, "mask": {"size": 7}},
          "mlp": _mlp(72, 1.5)},
         {"type": "rglru", "mixer": {"width": 48, "blocks": 3, "conv": 5}, "mlp": _mlp(40, 0.5)},
+        # of the rotated part's 12 dims only the first 8 turn
+        {"type": "latent_attention", "mixer": {"heads": 3, "dim": 16, "rot_dim": 12, "vdim": 8, "kv_rank": 20, "scale": 0.2,
+                                               "rot": {"base": 50.0, "dims": 8}}, "mlp": _mlp(40, 0.5)},
     ],
 }
 CONFIGS = {"P": CONFIG_P, "Q": CONFIG_Q}

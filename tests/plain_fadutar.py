@@ -124,14 +124,16 @@ def plain_latent_mixer(h: torch.Tensor, w: dict, prefix: str, mixer: dict, eps: 
     its latent vector, and the scores are sums over the unrotated and the rotated part."""
     tokens = h.shape[0]
     heads, dim, rot, vdim, rank = mixer["heads"], mixer["dim"], mixer["rot_dim"], mixer["vdim"], mixer["kv_rank"]
-    base = mixer["rot"]["base"]
-    assert mixer["rot"]["dims"] == rot
+    base, turn = mixer["rot"]["base"], mixer["rot"]["dims"]            # of the rot dims the first `turn` are rotated
     positions = torch.arange(tokens)
+
+    def rotated(part):
+        return torch.cat([plain_rotate_half(part[..., :turn], positions, base), part[..., turn:].double()], dim=-1)
     q = plain_linear(h, w[prefix + "q"]).reshape(tokens, heads, dim + rot)
-    q_plain, q_turned = q[..., :dim], plain_rotate_half(q[..., dim:], positions, base)
+    q_plain, q_turned = q[..., :dim], rotated(q[..., dim:])
     down = plain_linear(h, w[prefix + "dkv"])
     latent = plain_weight_norm(down[:, :rank], w[prefix + "dkv.norm"], eps)
-    k_turned = plain_rotate_half(down[:, rank:], positions, base)                  # [T, rot], one for all heads
+    k_turned = rotated(down[:, rank:])                                             # [T, rot], one for all heads
     k_plain = plain_linear(latent, w[prefix + "uk"]).reshape(tokens, heads, dim)
     values = plain_linear(latent, w[prefix + "uv"]).reshape(tokens, heads, vdim)
     out = torch.zeros((tokens, heads, vdim), dtype=torch.float64)

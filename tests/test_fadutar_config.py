@@ -54,7 +54,8 @@ def test_expected_tensors_follow_the_layers():
     (lambda raw: raw["layers"][1]["mixer"].update(kv_heads=4), "multiple"),
     (lambda raw: raw["layers"][0].update(type="lstm"), "not one of"),
     (lambda raw: raw["layers"][0]["mixer"].update(blocks=3), "multiple of blocks"),
-    (lambda raw: raw["layers"][3]["mixer"]["rot"].update(dims=6), "rot.dims"),
+    (lambda raw: raw["layers"][3]["mixer"]["rot"].update(dims=10), "rot.dims"),
+    (lambda raw: raw["layers"][3]["mixer"]["rot"].update(dims=3), "rot.dims"),
     (lambda raw: raw["layers"][1]["mlp"].update(kind="routed"), "dense"),
     (lambda raw: raw["norm"].pop("eps"), "eps"),
     (lambda raw: raw.pop("vocab"), "vocab"),

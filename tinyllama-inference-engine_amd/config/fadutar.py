@@ -10,7 +10,8 @@
     attention        heads, kv_heads, dim, vdim, scale, mask.size (a token sees its own chunk of so many
                      positions; no mask: every earlier position), kv_from (the layer whose keys and values
                      this one reads; it then has none of its own)
-    latent_attention heads, dim, rot_dim, vdim, kv_rank, scale, rot.base, rot.dims (= rot_dim)
+    latent_attention heads, dim, rot_dim, vdim, kv_rank, scale, rot.base, rot.dims (= rot_dim; fewer: the rest of
+                     the rot_dim part passes unrotated)
     rglru            width, blocks, conv (taps)
 
 Every size and every constant that can differ between two models of the design is read from here; what
@@ -112,8 +113,9 @@ class FadutarConfig:
         _number(where, mixer, "scale", float)
         rot = mixer.get("rot")
         _number(f"{where}'s rot", rot, "base", float)
-        if _number(f"{where}'s rot", rot, "dims") != rot_dim or rot_dim % 2 != 0:
-            raise invalid_config(f"{where}: rot.dims must equal rot_dim, and be even")
+        dims = _number(f"{where}'s rot", rot, "dims")
+        if dims > rot_dim or dims % 2 != 0:
+            raise invalid_config(f"{where}: rot.dims must be even and at most rot_dim (the dims past it pass unrotated)")
 
     def _check_rglru(self, index, mixer, where):
         width, blocks = _number(where, mixer, "width"), _number(where, mixer, "blocks")
@@ -180,7 +182,7 @@ class FadutarConfig:
             "hidden_size": width, "num_heads": int(mixer["heads"]), "head_dim": int(mixer["dim"]),
             "rot_dim": int(mixer["rot_dim"]), "value_dim": int(mixer["vdim"]), "rank": int(mixer["kv_rank"]),
             "scale": float(mixer["scale"]), "norm_eps": eps, "sink": True,
-            "position": PartSpec("rotary", {"head_dim": int(mixer["rot_dim"]), "theta": float(mixer["rot"]["base"]),
+            "position": PartSpec("rotary", {"head_dim": int(mixer["rot"]["dims"]), "theta": float(mixer["rot"]["base"]),
                                             "max_positions": None}),
             "names": {"q": "q", "down": "dkv", "down_norm": "dkv.norm", "up_keys": "uk", "up_values": "uv", "o": "o",
                       "sink": "sink"}})

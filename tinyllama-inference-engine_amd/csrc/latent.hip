@@ -14,7 +14,8 @@
 // the attention kernel that reads the page wants values as wide as keys; rows from rank on are never
 // written, and hold the zeros the pool was made with.
 //
-// Rotation: the pair (i, i + rot/2) by angle = float(position) * inv_freq[i], sines and cosines float.
+// Rotation: of a rotated part's first `turn` dims (turn <= rot, even; the rest pass unchanged) the pair
+// (i, i + turn/2) by angle = float(position) * inv_freq[i], sines and cosines float.
 // Norm: c = x * rsqrt(mean(x^2) + eps) * weight over the rank dims, in float.
 #include "common.h"
 
@@ -27,9 +28,9 @@ __global__ void latent_place_kernel(const D* __restrict__ fused, int nsplit, siz
                                     const int* __restrict__ positions, const int* __restrict__ slot_map,
                                     const float* __restrict__ inv_freq, const W* __restrict__ norm_weight, float eps,
                                     A* __restrict__ q_plain, A* __restrict__ q_wide, A* __restrict__ cache, int heads,
-                                    int plain, int rot, int rank, int value_rows, int page_size) {
+                                    int plain, int rot, int turn, int rank, int value_rows, int page_size) {
   extern __shared__ float lds[];
-  const int half = rot / 2;
+  const int half = turn / 2;
   float* cosines = lds;                  // half
   float* sines = cosines + half;         // half
   float* scratch = sines + half;         // 16
@@ -47,6 +48,7 @@ __global__ void latent_place_kernel(const D* __restrict__ fused, int nsplit, siz
 
   auto turned = [&](const D* part, int e) {        // element e of a rotated part that starts at `part`
     const float own = sum_splits(part + e, nsplit, split_stride);
+    if (e >= turn) return own;
     if (e < half) return own * cosines[e] - sum_splits(part + e + half, nsplit, split_stride) * sines[e];
     return own * cosines[e - half] + sum_splits(part + e - half, nsplit, split_stride) * sines[e - half];
   };
@@ -80,11 +82,12 @@ using namespace tlie;
 extern "C" int tlie_latent_place(const void* fused, int in_dtype, int nsplit, long long split_stride, const int* positions,
                                  const int* slot_map, const float* inv_freq, const void* norm_weight, int weight_dtype,
                                  float eps, void* q_plain, void* q_wide, void* cache, int act_dtype, int tokens, int heads,
-                                 int plain, int rot, int rank, int value_rows, int page_size, void* stream) {
-  if (tokens <= 0 || heads <= 0 || plain <= 0 || rot < 0 || rot % 2 != 0 || rank <= 0 || page_size <= 0 || nsplit < 1)
+                                 int plain, int rot, int turn, int rank, int value_rows, int page_size, void* stream) {
+  if (tokens <= 0 || heads <= 0 || plain <= 0 || rot < 0 || turn < 0 || turn > rot || turn % 2 != 0 || rank <= 0 || page_size <= 0 ||
+      nsplit < 1)
     return kBadArgument;
   if (value_rows != rank && value_rows != rank + rot) return kBadArgument;
-  if (rot > 0 && inv_freq == nullptr) return kBadArgument;
+  if (turn > 0 && inv_freq == nullptr) return kBadArgument;
   const int widest = heads * (plain + rot);
   const int threads = widest >= 1024 ? 1024 : (widest >= 256 ? 256 : 64);
   const size_t lds = (static_cast<size_t>(rot) + 16) * sizeof(float);
@@ -93,7 +96,7 @@ extern "C" int tlie_latent_place(const void* fused, int in_dtype, int nsplit, lo
   if (in_dtype == DC && weight_dtype == WC && act_dtype == AC) {                                                     \
     hipLaunchKernelGGL((latent_place_kernel<D, W, A>), dim3(tokens), dim3(threads), lds, s, (const D*)fused, nsplit,   \
                        (size_t)split_stride, positions, slot_map, inv_freq, (const W*)norm_weight, eps, (A*)q_plain,  \
-                       (A*)q_wide, (A*)cache, heads, plain, rot, rank, value_rows, page_size);                                   \
+                       (A*)q_wide, (A*)cache, heads, plain, rot, turn, rank, value_rows, page_size);                                   \
     return launch_status();                                                                                          \
   }
   TLIE_CASE(kF32, float, kF32, float, kF32, float)

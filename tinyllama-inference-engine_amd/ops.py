@@ -441,7 +441,7 @@ def block_linear(x: torch.Tensor, x_offset: int, x_row: int, x_block: int, weigh
 
 def latent_place(fused: Product, positions: torch.Tensor, slot_map: torch.Tensor, inv_freq: torch.Tensor | None,
                  norm_weight: torch.Tensor, eps: float, cache: torch.Tensor, heads: int, plain: int, rot: int, rank: int,
-                 act_dtype: torch.dtype, wide_values: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
+                 act_dtype: torch.dtype, wide_values: bool = False, turn: int | None = None) -> tuple[torch.Tensor, torch.Tensor]:
     """Latent attention between its first product and the attention kernel.  fused: [T, heads * (plain +
     rot) + rank + rot].  The rank dims are RMS-normed (weight, eps) and written to the cache rows of
     `slot_map` as keys [row][rank + rot] beside the rotated shared key part, and once more, transposed, as
@@ -449,7 +449,8 @@ def latent_place(fused: Product, positions: torch.Tensor, slot_map: torch.Tensor
     last rot dims, the rotated ones, are filled: the per-head product of q_plain fills the rest).
     wide_values: the value side of a page has rank + rot rows, as many as a key has dims (the cache is then
     [pages, 2, 1, page_size * (rank + rot)], what an attention kernel with one head size reads); its last rot
-    rows are never written."""
+    rows are never written.  turn: how many of the rot dims are rotated (the first ones; default all), inv_freq
+    then has turn / 2 entries."""
     _check_product(fused, "fused")
     _device_tensor(positions, "positions", torch.int32)
     _device_tensor(slot_map, "slot_map", torch.int32)
@@ -460,8 +461,9 @@ def latent_place(fused: Product, positions: torch.Tensor, slot_map: torch.Tensor
         raise invalid_shape(f"latent_place: width {fused.cols} is not heads * (plain + rot) + rank + rot")
     if positions.shape != (tokens,) or slot_map.shape != (tokens,):
         raise invalid_shape("latent_place: positions and slot_map need one entry per token")
-    if rot % 2 != 0 or rot < 0 or (rot > 0 and (inv_freq is None or inv_freq.shape != (rot // 2,))):
-        raise invalid_shape("latent_place: inv_freq needs rot / 2 entries, rot even")
+    turn = rot if turn is None else int(turn)
+    if rot < 0 or not 0 <= turn <= rot or turn % 2 != 0 or (turn > 0 and (inv_freq is None or inv_freq.shape != (turn // 2,))):
+        raise invalid_shape("latent_place: inv_freq needs one entry for every two rotated dims, an even number of them, at most rot")
     if inv_freq is not None:
         _device_tensor(inv_freq, "inv_freq", torch.float32)
     if not eps > 0.0:
@@ -472,7 +474,7 @@ def latent_place(fused: Product, positions: torch.Tensor, slot_map: torch.Tensor
     _check(library().tlie_latent_place(_ptr(fused.data), dtype_code(fused.data.dtype), fused.nsplit,
                                        ctypes.c_longlong(fused.split_stride), _ptr(positions), _ptr(slot_map), _ptr(inv_freq),
                                        _ptr(norm_weight), dtype_code(norm_weight.dtype), ctypes.c_float(eps), _ptr(q_plain),
-                                       _ptr(q_wide), _ptr(cache), dtype_code(act_dtype), tokens, heads, plain, rot, rank,
+                                       _ptr(q_wide), _ptr(cache), dtype_code(act_dtype), tokens, heads, plain, rot, turn, rank,
                                        rank + rot if wide_values else rank, page_size, _stream()), "latent_place")
     return q_plain, q_wide
 

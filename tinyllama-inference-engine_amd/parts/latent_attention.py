@@ -36,7 +36,8 @@ from .linear import Linear
 class LatentAttention(Mixer):
     """spec: hidden_size, num_heads, head_dim (a head's unrotated query/key dims), rot_dim (its rotated
     ones), value_dim, rank (of the latent vector), scale, norm_eps (of the latent vector's norm), sink (a
-    learned number per head in the softmax's denominator), position (a rotation table over rot_dim),
+    learned number per head in the softmax's denominator), position (a rotation table over the first dims of the
+    rot_dim part: all of them, or fewer, the rest then pass unchanged),
     names (the tensors' names after the prefix, by role).
     Tensors: q [H * (head_dim + rot_dim), hidden], down [rank + rot_dim, hidden], down_norm [rank],
     up_keys [H * head_dim, rank], up_values [H * value_dim, rank], o [hidden, H * value_dim], sink [H]."""
@@ -55,20 +56,20 @@ class LatentAttention(Mixer):
         self.scale = float(spec.get("scale") or 1.0 / math.sqrt(float(self.plain + self.rot)))
         self.norm_eps = float(spec["norm_eps"])
         self.has_sink = bool(spec.get("sink", False))
-        if min(self.heads, self.plain, self.dv, self.rank) <= 0 or self.rot < 0 or self.rot % 2 != 0:
-            raise invalid_config("latent_attention: sizes must be positive, rot_dim even")
+        if min(self.heads, self.plain, self.dv, self.rank) <= 0 or self.rot < 0:
+            raise invalid_config("latent_attention: sizes must be positive")
         if self.rank > ops.ATTENTION_MAX_HEAD_DIM:
             raise invalid_config(f"latent_attention: a latent vector of {self.rank} dims is beyond the attention kernel's "
                                  f"{ops.ATTENTION_MAX_HEAD_DIM} value dims")
         # values as wide as keys while that is a head size the attention kernels take
         self.wide_values = self.rank + self.rot <= ops.ATTENTION_MAX_HEAD_DIM
-        self.inv_freq = None
+        self.inv_freq, self.turn = None, 0             # turn: how many of the rot dims are rotated (the first ones)
         if self.rot > 0:
             position = spec["position"]
             table = lookup("position_encoding", position.kind)(position, dtype, device).rotary_table()
-            if table is None or table[1] != self.rot:
-                raise invalid_config("latent_attention: the position encoding must be a rotation table over rot_dim")
-            self.inv_freq = table[0]
+            if table is None or not 0 < table[1] <= self.rot:
+                raise invalid_config("latent_attention: the position encoding must be a rotation table over at most rot_dim dims")
+            self.inv_freq, self.turn = table
         self.names = {**self.NAMES, **dict(spec.get("names") or {})}
         self.first = self.o = self.down_norm = self.up_keys = self.up_values_t = self.sink = None
         self.up_keys_rows = self.up_values_rows = None
@@ -121,7 +122,7 @@ class LatentAttention(Mixer):
         tokens = fused.rows
         q_plain, q_wide = ops.latent_place(fused, ctx.positions, pages.slot_map if binding.writes else ctx.no_slots, self.inv_freq,
                                            self.down_norm, self.norm_eps, binding.cache, self.heads, self.plain, self.rot,
-                                           self.rank, self.dtype, wide_values=self.wide_values)
+                                           self.rank, self.dtype, wide_values=self.wide_values, turn=self.turn)
         ops.block_linear(q_plain, 0, self.heads * self.plain, self.plain, self.up_keys, None,
                          q_wide, 0, self.heads * key, key, tokens, weight=self.up_keys_rows)
         value_dim = key if self.wide_values else self.rank
