@@ -44,6 +44,12 @@ class LayerSpec:
     feed_forward_post_norm: PartSpec | None = None
     mixer_post_norm_place: str = "post_mixer_layernorm."
     feed_forward_post_norm_place: str = "post_feedforward_layernorm."
+    # for arrangements that scale what the sublayers add to the residual ("parallel"): the factor
+    residual_scale: float = 1.0
+    # something that joins the residual after the sublayers and depends on the step's tokens (a part of the
+    # "layer_input" table), and its place
+    layer_input: PartSpec | None = None
+    layer_input_place: str = "side."
 
 
 @dataclass(frozen=True)
@@ -57,6 +63,11 @@ class Run:
     """
     layer: int
     cache_of: int
+    # What joins the residual right before this run: the embedding's output once more, and row `add_vector[1]` of
+    # the tensor `add_vector[0]` ([rows, hidden]); for models that run a stretch of layers several times and
+    # tell the passes apart.
+    add_embedding: bool = False
+    add_vector: tuple[str, int] | None = None
 
 
 @dataclass(frozen=True)
@@ -81,6 +92,8 @@ class ModelSpec:
     # some writers store): regular expressions matched against the whole name.  Anything else that
     # the parts do not expect is an error.
     ignored_tensors: tuple[str, ...] = ()
+    # tensors that belong to no single part: tables that several layers read a part of each, the vectors that runs add
+    shared_tensors: tuple["TensorSpec", ...] = ()
 
     def validate(self) -> None:
         from ..errors import invalid_config
@@ -93,6 +106,11 @@ class ModelSpec:
                 raise invalid_config(f"run {index} reads the cache of run {run.cache_of}, which does not run before it")
             if self.runs[run.cache_of].cache_of != run.cache_of:
                 raise invalid_config(f"run {index} reads the cache of run {run.cache_of}, which owns none")
+            if run.add_vector is not None:
+                name, row = run.add_vector
+                shapes = [tensor.shape for tensor in self.shared_tensors if tensor.name == name]
+                if not shapes or len(shapes[0]) != 2 or shapes[0][1] != self.hidden_size or not 0 <= row < shapes[0][0]:
+                    raise invalid_config(f"run {index} adds row {row} of '{name}', which is no row of a shared tensor [rows, hidden]")
 
 
 @dataclass(frozen=True)

@@ -34,13 +34,21 @@ namespace tlie {
 // seq_start (or null) with min_tokens: the step's cumulative token counts per sequence; tokens of
 // sequences that bring min_tokens tokens or more are then left to the tiled kernel below, which
 // is launched beside this one for the same step and leaves the others to this one.
+// The attended values go out in the activation type, or, when the caller works on with them in 32-bit (two
+// maps of attention whose difference is normed), as floats: `out` then points to floats whatever T is.
+template <typename T>
+__device__ __forceinline__ void store_result(T* out, size_t index, float value, int out_f32) {
+  if (out_f32) reinterpret_cast<float*>(out)[index] = value;
+  else out[index] = from_float<T>(value);
+}
+
 template <typename T, int CHUNK>
 __global__ void __launch_bounds__(256)
 attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
                          int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
                          T* __restrict__ out, int nq, int nkv, int d, int dv, int page_size, int window, int chunk,
                          const float* __restrict__ sink, float scale,
-                         const int* __restrict__ seq_start, int min_tokens) {
+                         const int* __restrict__ seq_start, int min_tokens, int vshare, int out_f32) {
   constexpr int kGroups = 256 / CHUNK, kWavesPerGroup = CHUNK / 64;
   if (seq_start != nullptr) {                      // (the same for the whole workgroup)
     const int seq = token_seq[blockIdx.x];
@@ -60,9 +68,10 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
   const int* pages = block_table + static_cast<size_t>(token_seq[t]) * max_blocks;
   int lo = window > 0 ? max(0, pos - window + 1) : 0;
   if (chunk > 0) lo = max(lo, pos - pos % chunk);
-  const size_t page_stride = static_cast<size_t>(nkv) * page_size * (d + dv);
+  // (vshare key heads in a row read one value head: a page then holds nkv planes of keys and nkv / vshare of values)
+  const size_t page_stride = static_cast<size_t>(page_size) * (static_cast<size_t>(nkv) * d + static_cast<size_t>(nkv / vshare) * dv);
   const size_t head_offset = static_cast<size_t>(kv_head) * page_size * d;
-  const size_t v_offset = static_cast<size_t>(nkv) * page_size * d + static_cast<size_t>(kv_head) * page_size * dv;
+  const size_t v_offset = static_cast<size_t>(nkv) * page_size * d + static_cast<size_t>(kv_head / vshare) * page_size * dv;
 
   for (int i = threadIdx.x; i < d; i += 256) q_row[i] = to_float(q[(static_cast<size_t>(t) * nq + h) * d + i]);
   __syncthreads();
@@ -172,7 +181,7 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
       total += w * group_stat[2 * g + 1];
       result += w * group_out[g * dv + threadIdx.x];
     }
-    out[(static_cast<size_t>(t) * nq + h) * dv + threadIdx.x] = from_float<T>(result / total);
+    store_result(out, (static_cast<size_t>(t) * nq + h) * dv + threadIdx.x, result / total, out_f32);
   }
 }
 
@@ -195,7 +204,8 @@ __global__ void __launch_bounds__(64 * kTiledWaves)
 attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
                                int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
                                T* __restrict__ out, int tokens, int nq, int nkv, int d, int dv, int page_size, int window,
-                               int chunk, const float* __restrict__ sink, float scale, int tokens_per_block, int heads_per_block, const int* __restrict__ seq_start, int min_tokens) {
+                               int chunk, const float* __restrict__ sink, float scale, int tokens_per_block, int heads_per_block, const int* __restrict__ seq_start, int min_tokens,
+                               int vshare, int out_f32) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // rows of a multiple of 4 floats, so that four values are one LDS read, plus 4: a wave's lanes, each
   // on a row of its own, then spread over the banks
@@ -210,9 +220,10 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
   const int tok0 = blockIdx.x * tokens_per_block, head0 = blockIdx.z * heads_per_block;
   const int ntok = min(tokens_per_block, tokens - tok0), nheads = min(heads_per_block, G - head0);
   const int ncols = ntok * nheads;                 // column c = (token c / nheads, head c % nheads)
-  const size_t page_stride = static_cast<size_t>(nkv) * page_size * (d + dv);
+  // (vshare key heads in a row read one value head: a page then holds nkv planes of keys and nkv / vshare of values)
+  const size_t page_stride = static_cast<size_t>(page_size) * (static_cast<size_t>(nkv) * d + static_cast<size_t>(nkv / vshare) * dv);
   const size_t head_offset = static_cast<size_t>(kv_head) * page_size * d;
-  const size_t v_offset = static_cast<size_t>(nkv) * page_size * d + static_cast<size_t>(kv_head) * page_size * dv;
+  const size_t v_offset = static_cast<size_t>(nkv) * page_size * d + static_cast<size_t>(kv_head / vshare) * page_size * dv;
 
   for (int e = threadIdx.x; e < ncols * d; e += 64 * kTiledWaves) {
     const int c = e / d, i = e - c * d;
@@ -389,7 +400,7 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
         total += w * run_sum[g][s];
         result += w * acc[g][s];
       }
-      out[(static_cast<size_t>(tok0 + c / nheads) * nq + kv_head * G + head0 + c % nheads) * dv + lane] = from_float<T>(result / total);
+      store_result(out, (static_cast<size_t>(tok0 + c / nheads) * nq + kv_head * G + head0 + c % nheads) * dv + lane, result / total, out_f32);
     }
   }
 }
@@ -402,14 +413,14 @@ extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtyp
                                       int max_blocks, const int* token_seq, const int* positions, void* out,
                                       int tokens, int nq, int nkv, int d, int dv, int page_size, int window, int chunk,
                                       const float* sink, float scale, int tiled, const int* seq_start, int min_tokens,
-                                      void* stream) {
+                                      int vshare, int out_f32, void* stream) {
   // tiled 0: the kernel of one (token, head) a workgroup; 1: the kernel that shares keys among a
   // sequence's tokens (head sizes up to 64); 2: both, each token served by one of them: the second
   // takes the sequences that bring min_tokens tokens or more (seq_start: int32 [sequences + 1], the
   // step's cumulative token counts), the first the others.  A token gets the same bits from either.
   // (d only bounds the length of a dot product; dv is served by one thread a dim of a group of at most 256)
   if (tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 4096 || dv <= 0 || dv > 256 || page_size <= 0 ||
-      max_blocks <= 0 || chunk < 0)
+      max_blocks <= 0 || chunk < 0 || vshare <= 0 || nkv % vshare != 0)
     return kBadArgument;
   if (tiled < 0 || tiled > 2 || (tiled == 2 && (seq_start == nullptr || min_tokens < 1))) return kBadArgument;
   if (dtype != kF32 && dtype != kBF16) return kBadArgument;
@@ -426,11 +437,11 @@ extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtyp
     if (dtype == kF32)
       hipLaunchKernelGGL((attention_generic_tiled_kernel<float>), grid, dim3(64 * kTiledWaves), bytes, (hipStream_t)stream, (const float*)q,
                          (const float*)cache, block_table, max_blocks, token_seq, positions, (float*)out, tokens, nq, nkv, d, dv,
-                         page_size, window, chunk, sink, scale, tokens_per_block, heads_per_block, select, min_tokens);
+                         page_size, window, chunk, sink, scale, tokens_per_block, heads_per_block, select, min_tokens, vshare, out_f32);
     else
       hipLaunchKernelGGL((attention_generic_tiled_kernel<bf16>), grid, dim3(64 * kTiledWaves), bytes, (hipStream_t)stream, (const bf16*)q,
                          (const bf16*)cache, block_table, max_blocks, token_seq, positions, (bf16*)out, tokens, nq, nkv, d, dv,
-                         page_size, window, chunk, sink, scale, tokens_per_block, heads_per_block, select, min_tokens);
+                         page_size, window, chunk, sink, scale, tokens_per_block, heads_per_block, select, min_tokens, vshare, out_f32);
     const int status = launch_status();
     if (status != kOk || tiled == 1) return status;
   }
@@ -445,7 +456,7 @@ extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtyp
 #define TLIE_LAUNCH(T, CHUNK)                                                                                         \
   hipLaunchKernelGGL((attention_generic_kernel<T, CHUNK>), dim3(tokens, nq), dim3(256), lds, s, (const T*)q,           \
                      (const T*)cache, block_table, max_blocks, token_seq, positions, (T*)out, nq, nkv, d, dv, page_size, \
-                     window, chunk, sink, scale, select, min_tokens)
+                     window, chunk, sink, scale, select, min_tokens, vshare, out_f32)
   if (dtype == kF32) {
     if (keys == 64) TLIE_LAUNCH(float, 64); else if (keys == 128) TLIE_LAUNCH(float, 128); else TLIE_LAUNCH(float, 256);
   } else if (dtype == kBF16) {

@@ -147,22 +147,22 @@ template <typename D, typename A>
 __global__ void qkv_place_kernel(const D* __restrict__ qkv, int nsplit, size_t split_stride,
                                  const int* __restrict__ positions, const int* __restrict__ slot_map,
                                  const float* __restrict__ inv_freq, int rot_dim, A* __restrict__ q_out,
-                                 A* __restrict__ cache, int nq, int nkv, int d, int dv, int page_size) {
+                                 A* __restrict__ cache, int nq, int nkv, int nv, int d, int dv, int page_size, int row_width) {
   extern __shared__ float lds[];
   const int half = rot_dim / 2;
   float* cosines = lds;                  // half
   float* sines = cosines + half;         // half
   const int t = blockIdx.x;
-  const int rotated = (nq + nkv) * d, width = rotated + nkv * dv;
+  const int rotated = (nq + nkv) * d, width = rotated + nv * dv;
   if (inv_freq != nullptr) {
     const float pos = static_cast<float>(positions[t]);
     for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &sines[i], &cosines[i]);
     __syncthreads();
   }
   const int slot = nkv > 0 ? slot_map[t] : -1;
-  A* page = cache + static_cast<size_t>(slot < 0 ? 0 : slot / page_size) * nkv * page_size * (d + dv);
+  A* page = cache + static_cast<size_t>(slot < 0 ? 0 : slot / page_size) * page_size * (static_cast<size_t>(nkv) * d + static_cast<size_t>(nv) * dv);
   const int row = slot < 0 ? 0 : slot % page_size;
-  const D* in = qkv + static_cast<size_t>(t) * width;
+  const D* in = qkv + static_cast<size_t>(t) * row_width;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     if (c >= nq * d && slot < 0) break;  // (columns only grow: what is left is keys and values too)
     float v = sum_splits(in + c, nsplit, split_stride);
@@ -185,13 +185,18 @@ __global__ void qkv_place_kernel(const D* __restrict__ qkv, int nsplit, size_t s
 
 using namespace tlie;
 
-// q heads of d | k heads of d | v heads of dv; see qkv_place_kernel.
+// q heads of d | k heads of d | nv value heads of dv (nv = nkv, or fewer when several key heads share a value head:
+// a page then holds the nkv planes of keys and after them nv planes of values); a row of the product is
+// row_width columns long, of which these are the first.  See qkv_place_kernel.
 extern "C" int tlie_qkv_place(const void* qkv, int in_dtype, int nsplit, long long split_stride, const int* positions,
                               const int* slot_map, const float* inv_freq, int rot_dim, void* q_out, void* cache,
-                              int act_dtype, int tokens, int nq, int nkv, int d, int dv, int page_size, void* stream) {
+                              int act_dtype, int tokens, int nq, int nkv, int nv, int d, int dv, int page_size, int row_width,
+                              void* stream) {
   if (tokens <= 0 || nq <= 0 || nkv < 0 || d <= 0 || dv <= 0 || page_size <= 0 || nsplit < 1) return kBadArgument;
   if (rot_dim < 0 || rot_dim > d || rot_dim % 2 != 0 || (nkv > 0 && (cache == nullptr || slot_map == nullptr))) return kBadArgument;
-  const int width = (nq + nkv) * d + nkv * dv;
+  if (nv < 0 || nv > nkv || (nkv > 0 && (nv == 0 || nkv % nv != 0))) return kBadArgument;
+  const int width = (nq + nkv) * d + nv * dv;
+  if (row_width < width) return kBadArgument;
   const int threads = width >= 1024 ? 1024 : (width + 63) / 64 * 64;
   const size_t lds = static_cast<size_t>(rot_dim) * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
@@ -199,7 +204,7 @@ extern "C" int tlie_qkv_place(const void* qkv, int in_dtype, int nsplit, long lo
   if (in_dtype == DC && act_dtype == AC) {                                                                     \
     hipLaunchKernelGGL((qkv_place_kernel<D, A>), dim3(tokens), dim3(threads), lds, s, (const D*)qkv, nsplit,     \
                        (size_t)split_stride, positions, slot_map, inv_freq, rot_dim, (A*)q_out, (A*)cache, nq,  \
-                       nkv, d, dv, page_size);                                                                 \
+                       nkv, nv, d, dv, page_size, row_width);                                                                \
     return launch_status();                                                                                    \
   }
   TLIE_CASE(kF32, float, kF32, float)

@@ -1,0 +1,136 @@
+// Products with a handful of outputs whose sums are float whatever the types (a router's logits, the gates of a
+// recurrence), and what a routed feed-forward does with a router's scores.
+//
+//   few_outputs      out[t, n] = bias[n] + sum_k x[t, k] w[n, k]                          float out
+//   ... as a router  s = sigmoid(out[t, :]); the `top` largest s (the lower index wins a tie) keep their s,
+//                    all others become 0: scale[t, n]                                      float out
+//   routed_gate      hidden[t, c] = act(s g) * (s u), s = scale[t, c / block] for the first experts * block
+//                    columns and 1 for the rest (a shared expert's), g and u side by side in gate_up[t, 2c], [2c + 1]
+//
+// A token is a workgroup's: wave w of its four takes outputs w, w + 4, ..., lane l the inner indices l, l + 64,
+// ...: the order of a sum depends on the sizes alone.
+#include "common.h"
+
+namespace tlie {
+
+template <typename X, typename W>
+__global__ void __launch_bounds__(256)
+few_outputs_kernel(const X* __restrict__ x, const W* __restrict__ w, const W* __restrict__ bias, float* __restrict__ out,
+                   int inner, int outputs, int top) {
+  extern __shared__ float sums[];                      // outputs
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const X* row = x + static_cast<size_t>(t) * inner;
+  for (int n = wave; n < outputs; n += 4) {
+    const W* weights = w + static_cast<size_t>(n) * inner;
+    float a = 0.f, b = 0.f;
+    int k = lane;
+    for (; k + 64 < inner; k += 128) {
+      a += to_float(row[k]) * to_float(weights[k]);
+      b += to_float(row[k + 64]) * to_float(weights[k + 64]);
+    }
+    if (k < inner) a += to_float(row[k]) * to_float(weights[k]);
+    float total = wave_sum(a + b);
+    if (bias != nullptr) total += to_float(bias[n]);
+    if (top <= 0) {
+      if (lane == 0) out[static_cast<size_t>(t) * outputs + n] = total;
+    } else if (lane == 0) {
+      sums[n] = 1.f / (1.f + expf(-total));
+    }
+  }
+  if (top <= 0) return;
+  __syncthreads();
+  if (wave != 0) return;
+  // the first wave picks: `top` times the largest score that is left, the lower index on a tie
+  float* picked_out = out + static_cast<size_t>(t) * outputs;
+  for (int n = lane; n < outputs; n += 64) picked_out[n] = 0.f;
+  for (int round = 0; round < top; ++round) {
+    float best = -1.f;
+    int where = 1 << 30;
+    for (int n = lane; n < outputs; n += 64) {
+      const float s = sums[n];
+      if (s > best) best = s, where = n;               // (ascending n: the first of equals stays)
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+      const float other = __shfl_xor(best, offset, 64);
+      const int other_where = __shfl_xor(where, offset, 64);
+      if (other > best || (other == best && other_where < where)) best = other, where = other_where;
+    }
+    if (where >= outputs) break;                       // fewer outputs than `top`
+    if (lane == 0) {
+      picked_out[where] = best;
+      sums[where] = -2.f;
+    }
+    // lane 0's writes are ordered before the other lanes' next reads of sums[] (one wave: LDS operations complete in order)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+}
+
+template <typename D, typename A>
+__global__ void __launch_bounds__(256)
+routed_gate_kernel(const D* __restrict__ gate_up, int nsplit, size_t split_stride, const float* __restrict__ scale,
+                   int experts, int block, A* __restrict__ out, int inter) {
+  const int t = blockIdx.x;
+  const D* row = gate_up + static_cast<size_t>(t) * 2 * inter;
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < inter; c += gridDim.y * 256) {
+    const int e = c / block;
+    const float s = e < experts ? scale[static_cast<size_t>(t) * experts + e] : 1.f;
+    float v = 0.f;
+    if (s != 0.f) {                                    // an expert the token does not use: silu(0) * 0
+      const float g = s * sum_splits(row + 2 * c, nsplit, split_stride);
+      const float u = s * sum_splits(row + 2 * c + 1, nsplit, split_stride);
+      v = gated_value(g, u, kGateSilu, 1.f, 0.f);
+    }
+    out[static_cast<size_t>(t) * inter + c] = from_float<A>(v);
+  }
+}
+
+}  // namespace tlie
+
+using namespace tlie;
+
+// x: [tokens, inner] of x_dtype; w: [outputs, inner] and bias (or null) [outputs] of w_dtype; out: float [tokens, outputs].
+// top 0: the sums; top > 0: the router's scale matrix (see above).
+extern "C" int tlie_few_outputs(const void* x, int x_dtype, const void* w, const void* bias, int w_dtype, float* out,
+                                int tokens, int inner, int outputs, int top, void* stream) {
+  if (tokens <= 0 || inner <= 0 || outputs <= 0 || outputs > 4096 || top < 0) return kBadArgument;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t lds = static_cast<size_t>(outputs) * sizeof(float);
+#define TLIE_CASE(XC, X, WC, W)                                                                                       \
+  if (x_dtype == XC && w_dtype == WC) {                                                                               \
+    hipLaunchKernelGGL((few_outputs_kernel<X, W>), dim3(tokens), dim3(256), lds, s, (const X*)x, (const W*)w,          \
+                       (const W*)bias, out, inner, outputs, top);                                                     \
+    return launch_status();                                                                                           \
+  }
+  TLIE_CASE(kF32, float, kF32, float)
+  TLIE_CASE(kBF16, bf16, kBF16, bf16)
+  TLIE_CASE(kBF16, bf16, kF32, float)
+  TLIE_CASE(kF32, float, kBF16, bf16)
+#undef TLIE_CASE
+  return kBadArgument;
+}
+
+// gate_up: a product [nsplit][tokens][2 * inter], gate and up of a column side by side; scale: float [tokens, experts];
+// the first experts * block columns are the experts', the rest a shared expert's; out: [tokens, inter] of out_dtype.
+extern "C" int tlie_routed_gate(const void* gate_up, int in_dtype, int nsplit, long long split_stride, const float* scale,
+                                int experts, int block, void* out, int out_dtype, int tokens, int inter, void* stream) {
+  if (tokens <= 0 || inter <= 0 || experts < 0 || block <= 0 || nsplit < 1) return kBadArgument;
+  if (static_cast<long long>(experts) * block > inter) return kBadArgument;
+  int across = (inter + 255) / 256;
+  if (across > 64) across = 64;
+  const dim3 grid(tokens, across);
+  hipStream_t s = (hipStream_t)stream;
+#define TLIE_CASE(DC, D, AC, A)                                                                                       \
+  if (in_dtype == DC && out_dtype == AC) {                                                                            \
+    hipLaunchKernelGGL((routed_gate_kernel<D, A>), grid, dim3(256), 0, s, (const D*)gate_up, nsplit,                   \
+                       (size_t)split_stride, scale, experts, block, (A*)out, inter);                                  \
+    return launch_status();                                                                                           \
+  }
+  TLIE_CASE(kF32, float, kF32, float)
+  TLIE_CASE(kF32, float, kBF16, bf16)
+  TLIE_CASE(kBF16, bf16, kBF16, bf16)
+#undef TLIE_CASE
+  return kBadArgument;
+}

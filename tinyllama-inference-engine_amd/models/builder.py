@@ -10,6 +10,7 @@ from ..config.spec import ModelSpec, TensorSpec
 from .. import ops
 from ..ops import ResidualUpdated
 from ..registry import lookup
+from ..weights.arena import keep_in
 
 
 def expected_tensors(spec: ModelSpec) -> list[TensorSpec]:
@@ -21,6 +22,7 @@ def expected_tensors(spec: ModelSpec) -> list[TensorSpec]:
         specs += lookup("block", layer.block).tensor_specs(layer)
     specs += lookup("norm", spec.final_norm.kind).tensor_specs(spec.final_norm, spec.final_norm_prefix)
     specs += lookup("head", spec.head.kind).tensor_specs(spec.head, spec.head_name)
+    specs += list(spec.shared_tensors)
     names = [tensor.name for tensor in specs]
     if len(set(names)) != len(names):
         raise AssertionError("two parts claim the same tensor name")
@@ -39,6 +41,7 @@ class DecoderModel:
         self.blocks = [lookup("block", layer.block)(layer, dtype, device) for layer in spec.layers]
         self.final_norm = lookup("norm", spec.final_norm.kind)(spec.final_norm, dtype, device)
         self.head = lookup("head", spec.head.kind)(spec.head, dtype, device)
+        self.run_vectors: dict[str, torch.Tensor] = {}       # the tensors of which runs add a row to the residual, by name
 
     def load(self, weights) -> None:
         """weights: tensors on the device by name: a dict, or a `ResidentWeights`, which brings a
@@ -51,6 +54,10 @@ class DecoderModel:
             release()
         self.final_norm.load(weights, self.spec.final_norm_prefix)
         self.head.load(weights, self.spec.head_name)
+        for run in self.spec.runs:
+            if run.add_vector is not None and run.add_vector[0] not in self.run_vectors:
+                name = run.add_vector[0]
+                self.run_vectors[name] = keep_in(weights, weights[name].to(self.embedding.table.dtype).contiguous())
         release()
 
     @property
@@ -96,6 +103,13 @@ class DecoderModel:
             next_norm = entry_norm(self.blocks[runs[index + 1].layer]) if index + 1 < len(runs) else self.final_norm
             if trace is not None:
                 ctx.trace_prefix = f"layer{index}."
+            if run.add_embedding or run.add_vector is not None:
+                # what a run takes in before it starts: the residual is brought up to date first
+                if pending is not None and not isinstance(pending, ResidualUpdated):
+                    self._settle(residual, pending)
+                    pending = None
+                vector = self.run_vectors[run.add_vector[0]][run.add_vector[1]] if run.add_vector is not None else None
+                ops.residual_inject(residual, ctx.tokens, self.embedding.table if run.add_embedding else None, vector)
             pending = self.blocks[run.layer].forward(residual, pending, ctx, bindings[index], next_norm=next_norm)
         if ctx.num_wanted == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
@@ -110,6 +124,15 @@ class DecoderModel:
                 trace["final_norm"] = normed.float().clone()
             trace["logits"] = logits.clone()
         return logits
+
+
+    @staticmethod
+    def _settle(residual, pending) -> None:
+        """Adds what a block handed on into the residual now (a block whose result waits for the next norm)."""
+        if isinstance(pending, ops.NormedDelta):
+            ops.norm_add_rmsnorm(residual, pending.product, pending.weight, pending.eps, None, pending.eps, residual.dtype)
+        else:
+            residual += ops.as_product(pending).dense(torch.float32)
 
 
 def build_model(spec: ModelSpec, weights, dtype: torch.dtype, device) -> DecoderModel:

@@ -185,11 +185,22 @@ def silu_mul(gate_up: Product, out_dtype: torch.dtype, interleaved: bool = False
     return out
 
 
-def _check_cache(cache: torch.Tensor, num_kv_heads: int, head_dim: int, what: str, value_dim: int | None = None) -> int:
+def _check_cache(cache: torch.Tensor, num_kv_heads: int, head_dim: int, what: str, value_dim: int | None = None,
+                 value_heads: int | None = None) -> int:
     """cache: [pages, 2, nkv, page_size * d]; per page and kv head the keys lie as [row][dim] and
     the values transposed, [dim][row].  With a value size dv of its own a page is
     [nkv, page_size * (d + dv)] instead: the nkv planes of keys, then the nkv planes of values
-    (the same order of bytes when dv = d).  Returns the page size."""
+    (the same order of bytes when dv = d).  With fewer value heads than key heads (nkv / nv key heads in a
+    row read one value head) a page is [nv, page_size * (nkv / nv * d + dv)]: the nkv planes of keys, then
+    the nv planes of values.  Returns the page size."""
+    if value_heads is not None and value_heads != num_kv_heads:
+        dv = head_dim if value_dim is None else value_dim
+        if value_heads <= 0 or num_kv_heads % value_heads != 0:
+            raise invalid_shape(f"{what}: {num_kv_heads} key heads do not share {value_heads} value heads evenly")
+        per = num_kv_heads // value_heads * head_dim + dv
+        if cache.dim() != 3 or cache.shape[1] != value_heads or cache.shape[2] % per != 0:
+            raise invalid_shape(f"{what}: cache {list(cache.shape)} is not [pages, nv, page_size * (nkv / nv * d + dv)]")
+        return cache.shape[2] // per
     if value_dim is None or value_dim == head_dim:
         if cache.dim() != 4 or cache.shape[1] != 2 or cache.shape[2] != num_kv_heads or cache.shape[3] % head_dim != 0:
             raise invalid_shape(f"{what}: cache {list(cache.shape)} is not [pages, 2, nkv, page_size * d]")
@@ -251,7 +262,7 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
                       positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                       window: int | None, scale: float, tiled: bool | int = False, seq_start: torch.Tensor | None = None,
                       min_tokens: int = GENERIC_TILED_MIN_TOKENS, value_dim: int | None = None, chunk: int | None = None,
-                      sink: torch.Tensor | None = None) -> torch.Tensor:
+                      sink: torch.Tensor | None = None, value_heads: int | None = None, float_out: bool = False) -> torch.Tensor:
     """Causal attention of every token over its sequence's cached keys; any number of tokens per
     sequence.  block_table: [sequences, max_blocks] pages; token_seq[t]: the token's row of it.
     tiled 1 (True): the step's sequences bring several tokens each (consecutive in the step, at
@@ -263,9 +274,11 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
     value_dim: the size of a value head when it is not the key heads' (see `_check_cache`); the result is
     [tokens, nq * value_dim].  chunk: a token sees only the keys of its own chunk of so many positions
     (counted from position 0).  sink: float32 [nq], a number per head whose exponential joins the
-    softmax's denominator."""
+    softmax's denominator.  value_heads: fewer value heads than key heads (num_kv_heads / value_heads key heads in
+    a row read one value head; see `_check_cache`).  float_out: the result is float32 whatever q's type."""
     _device_tensor(q, "q", (torch.float32, torch.bfloat16))
     value_dim = head_dim if value_dim is None else int(value_dim)
+    value_heads = num_kv_heads if value_heads is None else int(value_heads)
     if sink is not None:
         _device_tensor(sink, "sink", torch.float32)
         if sink.shape != (num_heads,):
@@ -281,7 +294,7 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
     tokens = q.shape[0]
     if q.shape != (tokens, num_heads * head_dim):
         raise invalid_shape(f"attention: q {list(q.shape)} is not [tokens, nq * d]")
-    page_size = _check_cache(cache, num_kv_heads, head_dim, "attention", value_dim)
+    page_size = _check_cache(cache, num_kv_heads, head_dim, "attention", value_dim, value_heads)
     if block_table.dim() != 2 or token_seq.shape != (tokens,) or positions.shape != (tokens,):
         raise invalid_shape("attention: block_table must be [sequences, max_blocks], token_seq and positions [tokens]")
     if num_heads % num_kv_heads != 0:
@@ -293,13 +306,14 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
             raise invalid_shape("attention: seq_start needs one entry more than the block table has rows, min_tokens at least 1")
     elif tiled not in (0, 1):
         raise invalid_argument("attention: tiled is 0, 1 or 2")
-    out = torch.empty((tokens, num_heads * value_dim), dtype=q.dtype, device=q.device)
+    out = torch.empty((tokens, num_heads * value_dim), dtype=torch.float32 if float_out else q.dtype, device=q.device)
     _check(library().tlie_attention_generic(_ptr(q), _ptr(cache), dtype_code(q.dtype), _ptr(block_table),
                                             block_table.shape[1], _ptr(token_seq), _ptr(positions), _ptr(out), tokens,
                                             num_heads, num_kv_heads, head_dim, value_dim, page_size,
                                             int(window) if window else 0, int(chunk) if chunk else 0, _ptr(sink),
                                             ctypes.c_float(scale), tiled,
-                                            _ptr(seq_start if tiled == 2 else None), int(min_tokens), _stream()),
+                                            _ptr(seq_start if tiled == 2 else None), int(min_tokens),
+                                            num_kv_heads // value_heads, 1 if float_out else 0, _stream()),
            "attention_generic")
     return out
 
@@ -356,15 +370,18 @@ def norm_add_rmsnorm(residual: torch.Tensor, delta: Product, post_weight: torch.
 
 def qkv_place(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor | None, inv_freq: torch.Tensor | None,
               rot_dim: int, cache: torch.Tensor | None, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
-              act_dtype: torch.dtype) -> torch.Tensor:
+              act_dtype: torch.dtype, value_heads: int | None = None, extra_cols: int = 0) -> torch.Tensor:
     """`rope_cache` for any sizes: value heads of `value_dim` dims (a page is then nkv planes of keys and
     after them nkv planes of transposed values), and num_kv_heads 0 for a layer that reads another
-    layer's cache: only its queries [T, nq * d] are rotated and returned, nothing is written."""
+    layer's cache: only its queries [T, nq * d] are rotated and returned, nothing is written.
+    value_heads: fewer value heads than key heads (see `_check_cache`).  extra_cols: columns that the product
+    has after q, k and v, which are someone else's to read."""
     _check_product(qkv, "qkv")
     _device_tensor(positions, "positions", torch.int32)
     tokens = qkv.rows
-    if qkv.cols != (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim:
-        raise invalid_shape(f"qkv_place: qkv width {qkv.cols} is not (nq + nkv) * d + nkv * dv")
+    value_heads = num_kv_heads if value_heads is None else int(value_heads)
+    if extra_cols < 0 or qkv.cols != (num_heads + num_kv_heads) * head_dim + value_heads * value_dim + extra_cols:
+        raise invalid_shape(f"qkv_place: qkv width {qkv.cols} is not (nq + nkv) * d + nv * dv + {extra_cols}")
     if positions.shape != (tokens,):
         raise invalid_shape("qkv_place: positions need one entry per token")
     page_size = 1
@@ -373,7 +390,7 @@ def qkv_place(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor | No
         _device_tensor(cache, "cache", act_dtype)
         if slot_map.shape != (tokens,):
             raise invalid_shape("qkv_place: slot_map needs one entry per token")
-        page_size = _check_cache(cache, num_kv_heads, head_dim, "qkv_place", value_dim)
+        page_size = _check_cache(cache, num_kv_heads, head_dim, "qkv_place", value_dim, value_heads)
     if inv_freq is not None:
         _device_tensor(inv_freq, "inv_freq", torch.float32)
         if rot_dim % 2 != 0 or not 0 < rot_dim <= head_dim or inv_freq.shape != (rot_dim // 2,):
@@ -384,7 +401,8 @@ def qkv_place(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor | No
     _check(library().tlie_qkv_place(_ptr(qkv.data), dtype_code(qkv.data.dtype), qkv.nsplit, ctypes.c_longlong(qkv.split_stride),
                                     _ptr(positions), _ptr(slot_map if num_kv_heads > 0 else None), _ptr(inv_freq), rot_dim,
                                     _ptr(q_out), _ptr(cache if num_kv_heads > 0 else None), dtype_code(act_dtype), tokens,
-                                    num_heads, num_kv_heads, head_dim, value_dim, page_size, _stream()), "qkv_place")
+                                    num_heads, num_kv_heads, value_heads, head_dim, value_dim, page_size, qkv.cols, _stream()),
+           "qkv_place")
     return q_out
 
 
@@ -550,6 +568,213 @@ def gated_recurrence(fused: Product, x_col: int, y_col: int, u: torch.Tensor, ga
                                            _ptr(seq_slot), _ptr(out), dtype_code(out_dtype), seqs, channels, block_width,
                                            state.shape[1], slices, _ptr(parts), _stream()), "gated_recurrence")
     return out
+
+
+def head_combine(a: torch.Tensor, heads: int, value_dim: int, eps: float, out_dtype: torch.dtype, pair_group: int = 0,
+                 pair_lambda: float = 0.0, weight: torch.Tensor | None = None, mult: float = 1.0,
+                 gate: Product | None = None, gate_col: int = 0) -> torch.Tensor:
+    """Each head's result normed by itself, on its way to the output product:
+    out[t, h, :] = o / sqrt(mean(o^2) + eps) * weight[h] * mult * sigmoid(gate[t, h]), with o = a[t, h] or, for two maps
+    of attention a head (pair_group > 0: the query heads of one key head lie side by side in `a`, pair_group of them,
+    first all first maps' key heads ... see the kernel), o = first - pair_lambda * second.  a: float32
+    [tokens, heads (or 2 * heads) * value_dim]; weight (or None): [heads * value_dim]; gate (or None): a product whose
+    columns gate_col .. gate_col + heads * value_dim hold the gate's pre-activations."""
+    _device_tensor(a, "a", torch.float32)
+    maps = 2 if pair_group > 0 else 1
+    if a.dim() != 2 or a.shape[1] != maps * heads * value_dim:
+        raise invalid_shape(f"head_combine: a {list(a.shape)} is not [tokens, {maps} * heads * value_dim]")
+    if pair_group < 0 or (pair_group > 0 and heads % pair_group != 0):
+        raise invalid_shape("head_combine: the heads of a key head must divide the heads")
+    if not eps > 0.0:
+        raise EngineError(ErrorCode.NUMERICAL, "a norm requires a positive epsilon")
+    tokens = a.shape[0]
+    weight_code = F32
+    if weight is not None:
+        _device_tensor(weight, "weight", (torch.float32, torch.bfloat16))
+        if weight.shape != (heads * value_dim,):
+            raise invalid_shape("head_combine: the weight needs one entry per head and dim")
+        weight_code = dtype_code(weight.dtype)
+    gate_code, gate_nsplit, gate_stride, gate_row = F32, 1, 0, 0
+    if gate is not None:
+        _check_product(gate, "gate")
+        if gate.rows != tokens or gate_col < 0 or gate_col + heads * value_dim > gate.cols:
+            raise invalid_shape("head_combine: the gate's columns do not lie in the product")
+        gate_code, gate_nsplit, gate_stride, gate_row = dtype_code(gate.data.dtype), gate.nsplit, gate.split_stride, gate.cols
+    out = torch.empty((tokens, heads * value_dim), dtype=out_dtype, device=a.device)
+    if tokens == 0:
+        return out
+    _check(library().tlie_head_combine(_ptr(a), tokens, heads, value_dim, pair_group, ctypes.c_float(pair_lambda),
+                                       ctypes.c_float(eps), _ptr(weight), weight_code, ctypes.c_float(mult),
+                                       _ptr(gate.data if gate is not None else None), gate_code, gate_nsplit,
+                                       ctypes.c_longlong(gate_stride), gate_row, gate_col, _ptr(out), dtype_code(out_dtype),
+                                       _stream()), "head_combine")
+    return out
+
+
+MLSTM_MAX_DIM = 256            # the largest query/key size of a head that the matrix-memory kernel keeps in registers
+
+
+def mlstm_state_shape(heads: int, dim: int, value_dim: int) -> tuple[int, ...]:
+    """A request's state row for `mlstm_scan`: per head and tile of 64 value columns, S as [dim][64], n and m."""
+    return (heads, (value_dim + 63) // 64, dim * 64 + dim + 1)
+
+
+def mlstm_scan(fused: Product, q_col: int, k_col: int, v_col: int, gates: torch.Tensor, state: torch.Tensor,
+               seq_start: torch.Tensor, seq_slot: torch.Tensor, heads: int, dim: int, value_dim: int, cap: float,
+               q_scale: float) -> torch.Tensor:
+    """The matrix memory of an mLSTM layer over the step's tokens, sequence by sequence (see csrc/mlstm.hip): reads
+    q, k, v from the product's columns, the gates' pre-activations from `gates` (float32 [tokens, 2 * heads]: input
+    gates, then forget gates), carries `state` (float32 [slots, *mlstm_state_shape]) for sequences whose slot is not
+    negative, and returns float32 [tokens, heads * value_dim], the heads' results before their norm."""
+    _check_product(fused, "fused")
+    _device_tensor(gates, "gates", torch.float32)
+    _device_tensor(state, "state", torch.float32)
+    _device_tensor(seq_start, "seq_start", torch.int32)
+    _device_tensor(seq_slot, "seq_slot", torch.int32)
+    tokens = fused.rows
+    if not 0 < dim <= MLSTM_MAX_DIM or heads <= 0 or value_dim <= 0:
+        raise invalid_argument(f"mlstm_scan: heads of 1 to {MLSTM_MAX_DIM} query dims")
+    if gates.shape != (tokens, 2 * heads):
+        raise invalid_shape("mlstm_scan: the gates need two numbers a head and token")
+    if state.dim() != 4 or tuple(state.shape[1:]) != mlstm_state_shape(heads, dim, value_dim):
+        raise invalid_shape(f"mlstm_scan: state {list(state.shape)} is not [slots, {mlstm_state_shape(heads, dim, value_dim)}]")
+    sequences = seq_slot.shape[0]
+    if seq_start.shape != (sequences + 1,):
+        raise invalid_shape("mlstm_scan: seq_start needs one entry more than there are sequences")
+    for col, size in ((q_col, heads * dim), (k_col, heads * dim), (v_col, heads * value_dim)):
+        if col < 0 or col + size > fused.cols:
+            raise invalid_shape("mlstm_scan: q, k or v do not lie in the product's columns")
+    out = torch.empty((tokens, heads * value_dim), dtype=torch.float32, device=state.device)
+    if tokens == 0 or sequences == 0:
+        return out
+    _check(library().tlie_mlstm_scan(_ptr(fused.data), dtype_code(fused.data.dtype), fused.nsplit,
+                                     ctypes.c_longlong(fused.split_stride), fused.cols, q_col, k_col, v_col, _ptr(gates),
+                                     _ptr(state), _ptr(seq_start), _ptr(seq_slot), _ptr(out), sequences, heads, dim,
+                                     value_dim, ctypes.c_float(cap), ctypes.c_float(q_scale), _stream()), "mlstm_scan")
+    return out
+
+
+def few_outputs(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, top: int = 0) -> torch.Tensor:
+    """A product with few outputs and float sums: float32 [tokens, outputs] = x . weight^T + bias.  top > 0: as a
+    router: the sigmoids of the sums, of which each token's `top` largest keep their value and the rest become 0."""
+    _device_tensor(x, "x", (torch.float32, torch.bfloat16))
+    _device_tensor(weight, "weight", (torch.float32, torch.bfloat16))
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+        raise invalid_shape(f"few_outputs: x {list(x.shape)} does not fit weight {list(weight.shape)}")
+    outputs = weight.shape[0]
+    if outputs > 4096:
+        raise invalid_argument("few_outputs: at most 4096 outputs")
+    if bias is not None:
+        _device_tensor(bias, "bias", weight.dtype)
+        if bias.shape != (outputs,):
+            raise invalid_shape("few_outputs: the bias needs one entry per output")
+    if top < 0 or top > outputs:
+        raise invalid_argument("few_outputs: a router picks between 1 and all of its outputs")
+    out = torch.empty((x.shape[0], outputs), dtype=torch.float32, device=x.device)
+    if x.shape[0] == 0:
+        return out
+    _check(library().tlie_few_outputs(_ptr(x), dtype_code(x.dtype), _ptr(weight), _ptr(bias), dtype_code(weight.dtype),
+                                      _ptr(out), x.shape[0], x.shape[1], outputs, int(top), _stream()), "few_outputs")
+    return out
+
+
+def routed_gate(gate_up: Product, scale: torch.Tensor, block: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """hidden[t, c] = silu(s g) * (s u): g and u side by side in gate_up (g0 u0 g1 u1 ...), s = scale[t, c // block]
+    for the columns of the experts (scale: float32 [tokens, experts], 0 for an expert the token does not use) and 1
+    for the columns after them (an expert that every token uses)."""
+    _check_product(gate_up, "gate_up")
+    _device_tensor(scale, "scale", torch.float32)
+    if gate_up.cols % 2 != 0:
+        raise invalid_shape("routed_gate: gate and up lie side by side, the width must be even")
+    rows, inter = gate_up.rows, gate_up.cols // 2
+    if scale.dim() != 2 or scale.shape[0] != rows or block <= 0 or scale.shape[1] * block > inter:
+        raise invalid_shape("routed_gate: the scale matrix does not fit the columns")
+    out = torch.empty((rows, inter), dtype=out_dtype, device=gate_up.data.device)
+    if rows == 0:
+        return out
+    _check(library().tlie_routed_gate(_ptr(gate_up.data), dtype_code(gate_up.data.dtype), gate_up.nsplit,
+                                      ctypes.c_longlong(gate_up.split_stride), _ptr(scale), scale.shape[1], int(block),
+                                      _ptr(out), dtype_code(out_dtype), rows, inter, _stream()), "routed_gate")
+    return out
+
+
+@dataclass
+class SideInput:
+    """A per-layer token input for `residual_update`: the table [vocab, row] of which columns offset .. offset + dim
+    are the layer's, the gate [dim, width], the projection [width, dim], the norm's weight [width] and its eps."""
+    table: torch.Tensor
+    offset: int
+    dim: int
+    gate: torch.Tensor
+    proj: torch.Tensor
+    norm: torch.Tensor
+    eps: float
+
+
+RESIDUAL_UPDATE_MAX_WIDTH = 8000       # with a side input the kernel keeps two rows of floats in LDS
+
+
+def residual_update(residual: torch.Tensor, first: Product, second: Product | None, mult: float,
+                    side: SideInput | None = None, tokens: torch.Tensor | None = None) -> None:
+    """residual += mult * (first + second), in place; then, with `side`, the per-layer token input of the step's
+    `tokens` on the residual just brought up to date: g = gelu_tanh(gate x) * table[token, offset ..],
+    y = proj g, residual += mult * y / sqrt(mean(y^2) + eps) * norm."""
+    _device_tensor(residual, "residual", torch.float32)
+    _check_product(first, "first")
+    rows, width = residual.shape
+    products = [first] + ([second] if second is not None else [])
+    for product in products:
+        _check_product(product, "second")
+        if (product.rows, product.cols) != (rows, width) or product.data.dtype != first.data.dtype:
+            raise invalid_shape("residual_update: the sublayers' results do not fit the residual (or differ in type)")
+    if rows == 0:
+        return
+    args = [None, None, 0, 0, 0, None, None, None, F32, ctypes.c_float(1.0)]
+    if side is not None:
+        _device_tensor(tokens, "tokens", torch.int32)
+        for name in ("table", "gate", "proj", "norm"):
+            _device_tensor(getattr(side, name), name, side.table.dtype)
+        if (tokens.shape != (rows,) or side.table.dim() != 2 or side.offset < 0 or side.offset + side.dim > side.table.shape[1]
+                or side.gate.shape != (side.dim, width) or side.proj.shape != (width, side.dim) or side.norm.shape != (width,)):
+            raise invalid_shape("residual_update: the side input's tensors do not fit")
+        if width > RESIDUAL_UPDATE_MAX_WIDTH:
+            raise invalid_argument(f"residual_update: a side input goes with widths up to {RESIDUAL_UPDATE_MAX_WIDTH}")
+        if not side.eps > 0.0:
+            raise EngineError(ErrorCode.NUMERICAL, "a norm requires a positive epsilon")
+        args = [_ptr(tokens), _ptr(side.table), side.table.shape[1], side.offset, side.dim, _ptr(side.gate), _ptr(side.proj),
+                _ptr(side.norm), dtype_code(side.table.dtype), ctypes.c_float(side.eps)]
+    _check(library().tlie_residual_update(_ptr(residual), _ptr(first.data), first.nsplit, ctypes.c_longlong(first.split_stride),
+                                          _ptr(second.data if second is not None else None),
+                                          second.nsplit if second is not None else 1,
+                                          ctypes.c_longlong(second.split_stride if second is not None else 0),
+                                          dtype_code(first.data.dtype), ctypes.c_float(mult), rows, width, *args, _stream()),
+           "residual_update")
+
+
+def residual_inject(residual: torch.Tensor, tokens: torch.Tensor | None, table: torch.Tensor | None,
+                    vector: torch.Tensor | None, accumulate: bool = True) -> None:
+    """residual[t, :] (+)= table[tokens[t], :] + vector, in place; table and vector are optional and of one type."""
+    _device_tensor(residual, "residual", torch.float32)
+    rows, width = residual.shape
+    given = [tensor for tensor in (table, vector) if tensor is not None]
+    if not given:
+        if not accumulate:
+            residual.zero_()
+        return
+    code = dtype_code(given[0].dtype)
+    if table is not None:
+        _device_tensor(table, "table", given[0].dtype)
+        _device_tensor(tokens, "tokens", torch.int32)
+        if table.dim() != 2 or table.shape[1] != width or tokens.shape != (rows,):
+            raise invalid_shape("residual_inject: the table's rows are not the residual's, or tokens are missing")
+    if vector is not None:
+        _device_tensor(vector, "vector", given[0].dtype)
+        if vector.shape != (width,):
+            raise invalid_shape("residual_inject: the vector needs one entry per column")
+    if rows == 0:
+        return
+    _check(library().tlie_residual_inject(_ptr(residual), _ptr(tokens), _ptr(table), _ptr(vector), code, rows, width,
+                                          1 if accumulate else 0, _stream()), "residual_inject")
 
 
 def gemm_generic(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out_dtype: torch.dtype) -> Product:

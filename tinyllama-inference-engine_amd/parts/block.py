@@ -208,3 +208,77 @@ class SandwichNormBlock:
         ops.norm_add_rmsnorm(residual, out.product, out.weight, out.eps, None, out.eps, self.dtype)
         keep("output", residual)
         return None
+
+
+@register("block", "parallel")
+class ParallelBlock:
+    """x += scale * (mixer(norm(x)) + feed_forward(norm(x))): one norm, whose output both sublayers read; the
+    feed-forward is optional.  After that, if the layer has one, an input that depends on the step's tokens (a part
+    of the "layer_input" table) joins the residual.  The block brings the residual up to date itself, in one kernel
+    for the two results, their factor and the layer input, and hands on nothing."""
+
+    def __init__(self, layer: LayerSpec, dtype, device):
+        self.layer = layer
+        self.dtype = dtype
+        self.scale = float(layer.residual_scale)
+        self.mixer_norm = lookup("norm", layer.mixer_norm.kind)(layer.mixer_norm, dtype, device)
+        self.mixer = lookup("mixer", layer.mixer.kind)(layer.mixer, dtype, device)
+        self.feed_forward = self.layer_input = None
+        if layer.feed_forward is not None:
+            self.feed_forward = lookup("feed_forward", layer.feed_forward.kind)(layer.feed_forward, dtype, device)
+        if layer.layer_input is not None:
+            self.layer_input = lookup("layer_input", layer.layer_input.kind)(layer.layer_input, dtype, device)
+
+    @classmethod
+    def _parts(cls, layer: LayerSpec):
+        """(attribute, registry table) of the parts this layer has, in the order they run."""
+        parts = [("mixer_norm", "norm"), ("mixer", "mixer")]
+        if layer.feed_forward is not None:
+            parts.append(("feed_forward", "feed_forward"))
+        if layer.layer_input is not None:
+            parts.append(("layer_input", "layer_input"))
+        return parts
+
+    @classmethod
+    def tensor_specs(cls, layer: LayerSpec):
+        specs = []
+        for attribute, table in cls._parts(layer):
+            part_spec = getattr(layer, attribute)
+            specs += lookup(table, part_spec.kind).tensor_specs(part_spec, layer.prefix + getattr(layer, attribute + "_place"))
+        return specs
+
+    def load(self, weights):
+        for attribute, _ in self._parts(self.layer):
+            getattr(self, attribute).load(weights, self.layer.prefix + getattr(self.layer, attribute + "_place"))
+
+    def entry_norm(self):
+        return None
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(getattr(self, attribute), "graph_safe", False) for attribute, _ in self._parts(self.layer))
+
+    def forward(self, residual, pending, ctx, binding, next_norm=None):
+        """A step that keeps a trace leaves, under `ctx.trace_prefix`, "input_norm", "attention_output" (the mixer's
+        result), "mlp_output" (the feed-forward's, if there is one) and "output", the residual after the layer."""
+        trace = getattr(ctx, "trace", None)
+
+        def keep(name, tensor):
+            if trace is not None:
+                trace[ctx.trace_prefix + name] = tensor.float().clone()
+        normed = self.mixer_norm.add_forward(residual, pending)
+        keep("input_norm", normed)
+        mixed = as_product(self.mixer.forward(normed, ctx, binding))
+        if trace is not None:
+            keep("attention_output", mixed.dense(torch.float32))
+        fed = None
+        if self.feed_forward is not None:
+            fed = as_product(self.feed_forward.forward(normed, ctx))
+            if trace is not None:
+                keep("mlp_output", fed.dense(torch.float32))
+            if fed.data.dtype != mixed.data.dtype:       # (products of two kernels: as floats, so that one kernel adds both)
+                mixed, fed = ops.Product(mixed.dense(torch.float32).contiguous()), ops.Product(fed.dense(torch.float32).contiguous())
+        side = self.layer_input.side if self.layer_input is not None else None
+        ops.residual_update(residual, mixed, fed, self.scale, side=side, tokens=ctx.tokens if side is not None else None)
+        keep("output", residual)
+        return None

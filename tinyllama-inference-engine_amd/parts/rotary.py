@@ -14,7 +14,8 @@ from .base import PositionEncoding
 
 @register("position_encoding", "rotary")
 class Rotary(PositionEncoding):
-    """spec: head_dim, theta, optionally rot_dim (default head_dim: the whole head turns)."""
+    """spec: head_dim, theta, optionally rot_dim (default head_dim: the whole head turns) and linear_factor (every
+    frequency is divided by it: positions counted in steps of 1 / factor; default 1)."""
     graph_safe = True
 
     def __init__(self, spec: PartSpec, dtype, device):
@@ -26,9 +27,16 @@ class Rotary(PositionEncoding):
             raise invalid_config(f"rotary: rot_dim {self.rot_dim} must be even and at most head_dim {self.head_dim}")
         if not self.theta > 0:
             raise invalid_config("rotary: theta must be positive")
+        self.linear_factor = float(spec.get("linear_factor", 1.0))
+        if not self.linear_factor > 0:
+            raise invalid_config("rotary: linear_factor must be positive")
         index = torch.arange(self.rot_dim // 2, dtype=torch.float32)
         exponent = (-2.0 * index) / float(self.rot_dim)
-        self.inv_freq = torch.pow(torch.tensor(self.theta, dtype=torch.float32), exponent).to(device)
+        inv_freq = torch.pow(torch.tensor(self.theta, dtype=torch.float32), exponent)
+        if self.linear_factor != 1.0:
+            # formed in double and rounded once, so that the division costs the table no second rounding
+            inv_freq = (torch.pow(torch.tensor(self.theta, dtype=torch.float64), exponent.double()) / self.linear_factor).float()
+        self.inv_freq = inv_freq.to(device)
 
     def rotary_table(self):
         return self.inv_freq, self.rot_dim

@@ -19,9 +19,10 @@ POSITION_ENCODINGS: dict[str, Any] = {}
 BLOCKS: dict[str, Any] = {}
 EMBEDDINGS: dict[str, Any] = {}
 HEADS: dict[str, Any] = {}
+LAYER_INPUTS: dict[str, Any] = {}
 
 _TABLES = {"architecture": ARCHITECTURES, "mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
-           "position_encoding": POSITION_ENCODINGS, "block": BLOCKS, "embedding": EMBEDDINGS, "head": HEADS}
+           "position_encoding": POSITION_ENCODINGS, "block": BLOCKS, "embedding": EMBEDDINGS, "head": HEADS, "layer_input": LAYER_INPUTS}
 
 
 def register(table: str, name: str) -> Callable:
