@@ -87,16 +87,11 @@ def differential_attention(mixer, w, prefix, h, positions, eps):
 
 
 # ---- mLSTM ----------------------------------------------------------------------------------------------
-def mlstm(mixer, w, prefix, h, eps, state=None):
-    """h: [T, width] -> [T, width].  state: None (zeros) or (S [heads, dim, vdim], n [heads, dim], m [heads]);
-    the state after the last token is returned beside the output."""
-    heads, dim, vdim, cap = mixer["heads"], mixer["dim"], mixer["vdim"], float(mixer["gate_cap"])
-    T = h.shape[0]
-    q = (h @ w[prefix + "q"].T).reshape(T, heads, dim) * dim ** -0.5
-    k = (h @ w[prefix + "k"].T).reshape(T, heads, dim)
-    v = (h @ w[prefix + "v"].T).reshape(T, heads, vdim)
-    gate_i = cap * torch.tanh((h @ w[prefix + "i"].T + w[prefix + "i.b"]) / cap)
-    gate_f = torch.nn.functional.logsigmoid(cap * torch.tanh((h @ w[prefix + "f"].T + w[prefix + "f.b"]) / cap))
+def mlstm_memory(q, k, v, gate_i, gate_f, state=None):
+    """The matrix memory alone.  q, k: [T, heads, dim] (q scaled already), v: [T, heads, vdim], gate_i and gate_f: the log
+    gates [T, heads].  Returns the heads' results [T, heads, vdim] and the state (S, n, m) after the last token."""
+    T, heads, dim = q.shape
+    vdim = v.shape[-1]
     if state is None:
         S, n, m = torch.zeros(heads, dim, vdim, dtype=F64), torch.zeros(heads, dim, dtype=F64), torch.zeros(heads, dtype=F64)
     else:
@@ -111,8 +106,25 @@ def mlstm(mixer, w, prefix, h, eps, state=None):
         top = torch.einsum("hdv,hd->hv", S, q[t])
         bottom = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
         out[t] = top / bottom[:, None]
+    return out, (S, n, m)
+
+
+def log_gates(pre_i, pre_f, cap):
+    return cap * torch.tanh(pre_i / cap), torch.nn.functional.logsigmoid(cap * torch.tanh(pre_f / cap))
+
+
+def mlstm(mixer, w, prefix, h, eps, state=None):
+    """h: [T, width] -> [T, width].  state: None (zeros) or (S [heads, dim, vdim], n [heads, dim], m [heads]);
+    the state after the last token is returned beside the output."""
+    heads, dim, vdim, cap = mixer["heads"], mixer["dim"], mixer["vdim"], float(mixer["gate_cap"])
+    T = h.shape[0]
+    q = (h @ w[prefix + "q"].T).reshape(T, heads, dim) * dim ** -0.5
+    k = (h @ w[prefix + "k"].T).reshape(T, heads, dim)
+    v = (h @ w[prefix + "v"].T).reshape(T, heads, vdim)
+    gate_i, gate_f = log_gates(h @ w[prefix + "i"].T + w[prefix + "i.b"], h @ w[prefix + "f"].T + w[prefix + "f.b"], cap)
+    out, state = mlstm_memory(q, k, v, gate_i, gate_f, state)
     out = unit_rms(out, eps).reshape(T, heads * vdim) * w[prefix + "norm"] * torch.sigmoid(h @ w[prefix + "g"].T)
-    return out @ w[prefix + "o"].T, (S, n, m)
+    return out @ w[prefix + "o"].T, state
 
 
 # ---- feed-forwards --------------------------------------------------------------------------------------

@@ -118,5 +118,5 @@ class TensorSpec:
     """A tensor a part expects in the checkpoint: its full name, shape and kind of values."""
     name: str
     shape: tuple[int, ...]
-    init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "offset" (a norm's weight stored around 0), "zeros"
+    init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "offset" (a norm's weight stored around 0), "zeros", "forget_bias" (between 3 and 6)
     optional: bool = False       # absent is no error, present it is checked and not read (a tied head's matrix that some files still carry)

@@ -61,7 +61,8 @@ class MLSTM(Mixer):
                   ("gate", (heads * dv, hidden)), ("o", (hidden, heads * dv)), ("input_gate", (heads, hidden)),
                   ("forget_gate", (heads, hidden)))
         specs = [TensorSpec(prefix + names[role], shape) for role, shape in shapes]
-        specs += [TensorSpec(prefix + names[role], (heads,), init="zeros") for role in ("input_gate_bias", "forget_gate_bias")]
+        specs += [TensorSpec(prefix + names["input_gate_bias"], (heads,), init="zeros"),
+                  TensorSpec(prefix + names["forget_gate_bias"], (heads,), init="forget_bias")]
         specs.append(TensorSpec(prefix + names["norm"], (heads * dv,), init="norm"))
         return specs
 

@@ -43,6 +43,9 @@ def _draw(spec: TensorSpec, seed: int, std: float, norm_std: float, dtype: torch
         values = values * norm_std
     elif spec.init == "zeros":
         values = torch.zeros(spec.shape, device=device)
+    elif spec.init == "forget_bias":
+        # the bias of a forget gate, as such gates are commonly started: between 3 and 6, so that little is forgotten
+        values = 3.0 + 3.0 * torch.rand(spec.shape, generator=_generator(seed, spec.name + "#", device), dtype=torch.float32, device=device)
     else:
         raise ValueError(f"unknown init '{spec.init}' for {spec.name}")
     return values.to(dtype)
