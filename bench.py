@@ -197,20 +197,54 @@ def design_configs(sizes):
     return fadutar, llama
 
 
+# layer sizes for `--design raketar`: the same widths, feed-forwards and vocabulary; differential attention with half as many
+# heads of two maps each (so that its query heads are Llama's) and values twice as wide; memory heads after the ratios
+# of published xLSTM models (query/key half as wide as the values); routed feed-forwards whose experts in use plus the
+# shared one are as wide as the dense feed-forward; four layers of which the first two run twice (six runs)
+RAKETAR_SIZES = {
+    "w2048": dict(width=2048, ff=5632, heads=16, kv_heads=2, dim=64, vdim=128, memory_heads=8, memory_dim=128, memory_vdim=256,
+                  experts=8, top=2, expert_ff=1408, shared_ff=2816, side=128, vocab=32000, llama_heads=32, llama_kv_heads=4),
+    "w4096": dict(width=4096, ff=14336, heads=16, kv_heads=4, dim=128, vdim=256, memory_heads=8, memory_dim=256, memory_vdim=512,
+                  experts=8, top=2, expert_ff=3584, shared_ff=7168, side=128, vocab=32000, llama_heads=32, llama_kv_heads=8),
+}
+
+
+def raketar_configs(sizes):
+    """(the Raketar configuration, the Llama configuration of equal sizes): differential attention with a dense
+    feed-forward, a memory layer with a routed one, differential attention with a routed one, a memory layer with a
+    dense one; the first two run twice.  Beside as many Llama layers as that makes runs."""
+    s = sizes
+    dense = {"kind": "dense", "ff": s["ff"]}
+    routed = {"kind": "moe", "expert": {"ff": s["expert_ff"]}, "router": {"experts": s["experts"], "top": s["top"]},
+              "shared": {"ff": s["shared_ff"]}}
+    attention = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["vdim"], "scale": s["dim"] ** -0.5,
+                 "diff": 0.5, "rot": {"base": 10000.0, "dims": s["dim"], "scaling": {"factor": 2.0}}}
+    memory = {"heads": s["memory_heads"], "dim": s["memory_dim"], "vdim": s["memory_vdim"], "gate_cap": 15.0}
+    layers = [{"type": "attention", "mixer": attention, "mlp": dense}, {"type": "mlstm", "mixer": memory, "mlp": routed},
+              {"type": "attention", "mixer": attention, "mlp": routed}, {"type": "mlstm", "mixer": memory, "mlp": dense}]
+    raketar = {"architecture": "Raketar", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+               "token_side": {"dim": s["side"]}, "loop": {"start": 0, "stop": 2, "times": 2}, "layers": layers}
+    llama = dict(TINYLLAMA, hidden_size=s["width"], intermediate_size=s["ff"], num_hidden_layers=6,
+                 num_attention_heads=s["llama_heads"], num_key_value_heads=s["llama_kv_heads"], vocab_size=s["vocab"],
+                 max_position_embeddings=4096)
+    return raketar, llama
+
+
 def bench_design(args, torch) -> int:
-    """`--design fadutar`: one JSON line.  Per size: tokens a second of a prompt step of 2048 tokens and of decode steps
-    at the record's batch and context, for the Fadutar decoder and for the Llama decoder of equal sizes (random
+    """`--design fadutar|raketar`: one JSON line.  Per size: tokens a second of a prompt step of 2048 tokens and of decode steps
+    at the record's batch and context, for that decoder and for the Llama decoder of equal sizes (random
     weights, bfloat16, through the engine's own loop), and every kernel the design adds alone, beside the like kernel."""
     from tlie_amd import Engine, ops
-    from tlie_amd.kernel_bench import bench_design_kernels
+    from tlie_amd.kernel_bench import bench_design_kernels, bench_raketar_kernels
     peaks = ops.measured_peaks("cuda:0")
     record = {"metric": f"{args.design}: prefill and decode tok/s beside the Llama decoder of equal sizes", "unit": "tokens/s",
               "n_gpus": 1, "dtype": "bf16", "data": "synthetic: uniform random token ids, random weights",
               "batch": args.batch, "context": args.context, "measured_peaks": peaks, "sizes": {}}
     steps, warmup = min(args.steps, 48), 4
-    for name, sizes in DESIGN_SIZES.items():
-        entry = {"layers": 4 * sizes["groups"], "sizes": sizes}
-        for model, config in zip(("fadutar", "llama"), design_configs(sizes)):
+    all_sizes, configs = (DESIGN_SIZES, design_configs) if args.design == "fadutar" else (RAKETAR_SIZES, raketar_configs)
+    for name, sizes in all_sizes.items():
+        entry = {"layers": 4 * sizes["groups"] if args.design == "fadutar" else 6, "sizes": sizes}
+        for model, config in zip((args.design, "llama"), configs(sizes)):
             engine = Engine(None, dtype="bfloat16", config=config, random_seed=0, max_tokens=args.batch * args.context + 4096,
                             page_size=16, max_requests=args.batch + 1)
             seconds = time_prefill(engine, torch, 2048, sizes["vocab"])
@@ -221,8 +255,10 @@ def bench_design(args, torch) -> int:
             entry[f"{model}_decode_ms_step"] = seconds / steps * 1e3
             del engine
             torch.cuda.empty_cache()
-        entry["kernels"] = bench_design_kernels(sizes, batch=args.batch, context=args.context, prompt=2048,
-                                                hbm_gbs=peaks["stream_read_gbs"], mfma_tflops=peaks["mfma_bf16_tflops"])
+        kernels = bench_design_kernels if args.design == "fadutar" else bench_raketar_kernels
+        if not args.no_points:
+            entry["kernels"] = kernels(sizes, batch=args.batch, context=args.context, prompt=2048,
+                                       hbm_gbs=peaks["stream_read_gbs"], mfma_tflops=peaks["mfma_bf16_tflops"])
         record["sizes"][name] = entry
     record["library_fallbacks"] = ops.library_fallbacks()
     print(json.dumps(record))
@@ -254,7 +290,7 @@ def main() -> int:
                         help="time the kernels of a decode step (--batch, --context) and of a prompt step one by one at the "
                              "shape's layer sizes, each inside a replayed recording that walks through copies of its weights; "
                              "NAME keeps the kernels whose name holds it; prints one JSON line per kernel")
-    parser.add_argument("--design", default=None, choices=["fadutar"],
+    parser.add_argument("--design", default=None, choices=["fadutar", "raketar"],
                         help="prefill and decode throughput of that decoder design at layer sizes of real models, beside the Llama "
                              "decoder at equal sizes, and its own kernels alone beside the like kernels (one JSON line of its own)")
     parser.add_argument("--shape", default="tinyllama", choices=["tinyllama", *OTHER_SHAPES],

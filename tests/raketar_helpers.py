@@ -53,7 +53,8 @@ CONFIG_T = {        # no loop; a single layer of each kind
     "architecture": "Raketar", "vocab": 64, "width": 32, "norm": {"eps": 1e-5}, "residual_mult": 0.25, "token_side": {"dim": 3},
     "layers": [
         {"type": "mlstm", "mixer": {"heads": 2, "dim": 8, "vdim": 70, "gate_cap": 6.0}, "mlp": None},
-        {"type": "attention", "mixer": _attention(2, 1, 12, 16, 0.3, 0.6, {"base": 100.0, "dims": 4, "scaling": {"factor": 1.5}}),
+        # values twice as wide as the keys, both multiples of 16: in bfloat16 this layer takes the kernel on the matrix cores
+        {"type": "attention", "mixer": _attention(4, 2, 16, 32, 0.3, 0.6, {"base": 100.0, "dims": 4, "scaling": {"factor": 1.5}}),
          "mlp": _moe(4, 2, 8, 8)},
     ],
 }

@@ -83,6 +83,13 @@ def test_two_maps_are_combined_normed_and_gated(heads, per_group, dv, nsplit):
                            pair_group=per_group, pair_lambda=lam, mult=mult, gate=split_product(gate, nsplit, generator), gate_col=11)
     want = plain.unit_rms(first.double() - lam * second.double(), eps) * mult * torch.sigmoid(gate[:, 11:].double()).reshape(tokens, heads, dv)
     assert float((got.cpu().double() - want.reshape(tokens, -1)).abs().max()) < 2e-5
+    # a map's result in pieces, each a head of its own of the attention kernel: (key head, piece, query head of the key head)
+    for parts in (2, 3, 5):
+        if dv % parts == 0:
+            pieces = a.reshape(tokens, 2 * groups, per_group, parts, dv // parts).transpose(2, 3).contiguous()
+            again = ops.head_combine(pieces.reshape(tokens, -1).to(DEVICE), heads, dv, eps, torch.float32, pair_group=per_group,
+                                     pair_lambda=lam, mult=mult, gate=split_product(gate, 1, generator), gate_col=11, parts=parts)
+            assert float((again - got).abs().max()) < 1e-6
     # one result a head, with a weight, in bfloat16 out
     weight = torch.randn(heads * dv, generator=generator)
     got = ops.head_combine(first.reshape(tokens, -1).contiguous().to(DEVICE), heads, dv, eps, torch.bfloat16, weight=weight.to(DEVICE))
@@ -314,11 +321,13 @@ def _mixer_alone(folder, tokens, dtype, cuts):
     {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.3, "diff": 0.3, "rot": {"base": 1000.0, "dims": 8, "scaling": {"factor": 2.0}}},
     {"heads": 3, "kv_heads": 1, "dim": 6, "vdim": 70, "scale": 0.5, "diff": 0.7, "rot": {"base": 20.0, "dims": 6}},
     {"heads": 2, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 0.2, "diff": 0.5, "rot": {"base": 250000.0, "dims": 32, "scaling": {"factor": 4.0}}},
+    {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 48, "scale": 0.25, "diff": 0.2, "rot": {"base": 300.0, "dims": 8}},
+    {"heads": 6, "kv_heads": 1, "dim": 64, "vdim": 128, "scale": 0.125, "diff": 0.5, "rot": {"base": 10000.0, "dims": 64}},
 ])
 def test_differential_attention_alone(tmp_path, mixer, dtype):
     folder, config, weights = _single_layer(tmp_path, {"type": "attention", "mixer": mixer, "mlp": None}, seed=5)
-    tokens = tokens_of(6, 90, 97)
-    for cuts in ([90], [33, 1, 2, 20], [1]):
+    tokens = tokens_of(6, 300, 97)             # (long enough for the keys to be cut into parts that are merged)
+    for cuts in ([300], [33, 1, 2, 20, 150], [280] + [1] * 20):
         h, got = _mixer_alone(folder, tokens, dtype, cuts)
         want = plain.differential_attention(mixer, weights, "l0.mix.", h, torch.arange(len(tokens)), 1e-5)
         assert_rows(got, want, 2e-5 if dtype == "float32" else 3e-2, f"cuts {cuts}")

@@ -105,7 +105,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
                       const int* __restrict__ block_table, int max_blocks, const int4* __restrict__ tiles,
                       const int* __restrict__ positions, uint16_t* __restrict__ out, float* __restrict__ part_o,
                       float* __restrict__ part_ml, int nsplit, int split_len, int nq, int nkv, int page_size,
-                      int window, int chunk, const float* __restrict__ sink, float scale_log2, int round_size) {
+                      int window, int chunk, const float* __restrict__ sink, float scale_log2, int round_size, int plane_map) {
   constexpr int D = DT * 16;
   // the first key that the token at position p sees: the window's edge, or the start of the token's own
   // chunk of positions (chunks are counted from position 0), whichever is later; 0 without either
@@ -154,14 +154,30 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   const int group_col0 = col0;                                   // the workgroup's first column
   if (SHARED) col0 += __builtin_amdgcn_readfirstlane(wave) * 16 * CT;
   const bool wave_active = col0 < ncols;                         // (a shared tile's last waves may have no column)
+  // Which planes of a page the kv head reads: its own key and value plane, or (EXTRA, plane_map != 0) planes that
+  // several kv heads share: kdiv kv heads in a row read one key plane, and of every vgroup kv heads in a row the
+  // i-th reads value plane i % vmod of the group's vmod: a page then holds nkv / kdiv planes of keys and after them
+  // nkv / vgroup * vmod planes of values, and q holds one query head for the kv heads that share a key plane (a
+  // value head wider than the keys, cut into parts of the keys' size, each part a kv head of the kernel's; two maps
+  // of attention that read the same values).  Bit 24: the results go out as floats.
+  int k_plane = kvh, v_plane = kvh, planes_k = nkv, planes_v = nkv;
+  bool float_out = false;
+  if (EXTRA && plane_map != 0) {
+    const int kdiv = plane_map & 255, vgroup = (plane_map >> 8) & 255, vmod = (plane_map >> 16) & 255;
+    float_out = (plane_map >> 24) & 1;
+    k_plane = kvh / kdiv, v_plane = (kvh / vgroup) * vmod + kvh % vmod;
+    planes_k = nkv / kdiv, planes_v = nkv / vgroup * vmod;
+  }
+  const int nq_in = planes_k * G;                                // query heads a token has in q
   bool valid_col[CT];
-  int tok[CT], head[CT], pos_col[CT], lo_col[CT];
+  int tok[CT], head[CT], q_head[CT], pos_col[CT], lo_col[CT];
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
     const int c = col0 + ct * 16 + col;
     valid_col[ct] = c < ncols;
     tok[ct] = tok0 + (valid_col[ct] ? c / G : 0);
     head[ct] = kvh * G + (valid_col[ct] ? c % G : 0);
+    q_head[ct] = k_plane * G + (valid_col[ct] ? c % G : 0);
     pos_col[ct] = valid_col[ct] ? pos0 + c / G : -1;
     lo_col[ct] = bounded ? lower(pos_col[ct]) : 0;
   }
@@ -196,9 +212,9 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
     return place < 64 ? low : high;                        // (all scalar: a select, not a mask)
   };
   const int table_span = 128 << page_shift;                // keys that one window covers
-  const size_t page_stride = static_cast<size_t>(2) * nkv * page_size * D;
-  const uint16_t* k_base = cache + static_cast<size_t>(kvh) * page_size * D;
-  const uint16_t* v_base = k_base + static_cast<size_t>(nkv) * page_size * D;
+  const size_t page_stride = static_cast<size_t>(planes_k + planes_v) * page_size * D;
+  const uint16_t* k_base = cache + static_cast<size_t>(k_plane) * page_size * D;
+  const uint16_t* v_base = cache + static_cast<size_t>(planes_k + v_plane) * page_size * D;
   const int k_lane = col * D + grp * 8;                    // operand A of the first product: key `col`, dims grp*8..
   const int v_lane = (col << page_shift) + grp * 4;        // operand A of the second: dim `col`, keys grp*4..
 
@@ -211,7 +227,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
       const int dim = ks * 32 + grp * 8;
       qreg[ct][ks].u = make_uint4(0, 0, 0, 0);
       if (valid_col[ct] && has_dims(ks))
-        qreg[ct][ks].u = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(tok[ct]) * nq + head[ct]) * D + dim);
+        qreg[ct][ks].u = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(tok[ct]) * nq_in + q_head[ct]) * D + dim);
     }
 
   // The softmax runs in base 2: scores are scaled by scale * log2(e) and exponentiated with exp2
@@ -574,6 +590,14 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
         inv = mine / (running_sum[ct] * mine + __builtin_amdgcn_exp2f(own - top));
       }
       uint16_t* o_row = out + (static_cast<size_t>(tok[ct]) * nq + head[ct]) * D;
+      if (EXTRA && float_out) {
+        float* f_row = reinterpret_cast<float*>(out) + (static_cast<size_t>(tok[ct]) * nq + head[ct]) * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          *reinterpret_cast<float4*>(f_row + dt * 16 + grp * 4) =
+              make_float4(o[ct][dt][0] * inv, o[ct][dt][1] * inv, o[ct][dt][2] * inv, o[ct][dt][3] * inv);
+        continue;
+      }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         uint2 packed;
@@ -602,7 +626,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
 // the weights are formed once, by the lanes, and kept in LDS.
 __global__ void __launch_bounds__(64)
 attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                       uint16_t* __restrict__ out, int nsplit, int d, const float* __restrict__ sink, int nq) {
+                       uint16_t* __restrict__ out, int nsplit, int d, const float* __restrict__ sink, int nq, int float_out) {
   extern __shared__ float weight[];                  // nsplit
   const size_t row = blockIdx.x;                     // token * nq + head
   const float* ml = part_ml + row * nsplit * 2;
@@ -646,7 +670,10 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
         a += weight[p] * early[p];
       }
     }
-    if (lane < d) out[row * d + lane] = __bfloat16_as_ushort(__float2bfloat16((a + b) * inv));
+    if (lane < d) {
+      if (float_out) reinterpret_cast<float*>(out)[row * d + lane] = (a + b) * inv;
+      else out[row * d + lane] = __bfloat16_as_ushort(__float2bfloat16((a + b) * inv));
+    }
     return;
   }
   for (int i = lane; i < d; i += 64) {
@@ -658,7 +685,8 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
       b += weight[p + 1] * column[static_cast<size_t>(p + 1) * d];
     }
     if (p < nsplit) a += weight[p] * column[static_cast<size_t>(p) * d];
-    out[row * d + i] = __bfloat16_as_ushort(__float2bfloat16((a + b) * inv));
+    if (float_out) reinterpret_cast<float*>(out)[row * d + i] = (a + b) * inv;
+    else out[row * d + i] = __bfloat16_as_ushort(__float2bfloat16((a + b) * inv));
   }
 }
 
@@ -679,19 +707,19 @@ template <int DT, int CT, bool SHARED = false>
 static int launch_attention(const void* q, const void* cache, const int* block_table, int max_blocks, const void* tiles,
                             int num_tiles, const int* positions, void* out, float* part_o, float* part_ml, int nsplit,
                             int split_len, int nq, int nkv, int page_size, int window, int chunk, const float* sink, float scale,
-                            int waves, hipStream_t stream) {
+                            int waves, hipStream_t stream, int plane_map) {
   const float scale_log2 = scale * 1.4426950408889634f;
   // LDS for merging the waves: their maxima and sums, and half as many slots as waves for the results
   const size_t lds = !SHARED && waves > 1 ? (static_cast<size_t>(waves) * CT * 32 + static_cast<size_t>(waves / 2) * CT * DT * 256) * sizeof(float) : 0;
   if (lds > 64 * 1024) return kBadArgument;
-  if (chunk > 0 || sink != nullptr)
+  if (chunk > 0 || sink != nullptr || plane_map != 0)
     hipLaunchKernelGGL((attention_mfma_kernel<DT, CT, SHARED, true>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
                        (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
-                       part_ml, nsplit, split_len, nq, nkv, page_size, window, chunk, sink, scale_log2, compute_units());
+                       part_ml, nsplit, split_len, nq, nkv, page_size, window, chunk, sink, scale_log2, compute_units(), plane_map);
   else
     hipLaunchKernelGGL((attention_mfma_kernel<DT, CT, SHARED, false>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
                        (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
-                       part_ml, nsplit, split_len, nq, nkv, page_size, window, 0, nullptr, scale_log2, compute_units());
+                       part_ml, nsplit, split_len, nq, nkv, page_size, window, 0, nullptr, scale_log2, compute_units(), 0);
   return launch_status();
 }
 
@@ -713,8 +741,13 @@ static int attention_entry(const void* q, const void* cache, const int* block_ta
                            const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
                            float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
                            int d, int page_size, int window, int chunk, const float* sink, float scale, int waves, int shared,
-                           void* stream) {
+                           void* stream, int plane_map = 0) {
   if (chunk < 0) return kBadArgument;
+  if (plane_map != 0) {
+    const int kdiv = plane_map & 255, vgroup = (plane_map >> 8) & 255, vmod = (plane_map >> 16) & 255;
+    if (kdiv <= 0 || vgroup <= 0 || vmod <= 0 || vmod > vgroup || nkv % kdiv != 0 || nkv % vgroup != 0 || (plane_map >> 25) != 0)
+      return kBadArgument;
+  }
   if (num_tiles <= 0 || tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 256 || d % 16 != 0 ||
       page_size < 16 || (page_size & (page_size - 1)) != 0 || max_blocks <= 0 || nsplit < 1 || nsplit > 65535 || nkv > 65535)
     return kBadArgument;
@@ -731,7 +764,7 @@ static int attention_entry(const void* q, const void* cache, const int* block_ta
   hipStream_t s = (hipStream_t)stream;
   int status = kBadArgument;
 #define TLIE_ARGS q, cache, block_table, max_blocks, tiles, num_tiles, positions, out, part_o, part_ml, nsplit, split_len, nq, \
-                  nkv, page_size, window, chunk, sink, scale, waves, s
+                  nkv, page_size, window, chunk, sink, scale, waves, s, plane_map
 #define TLIE_CASE(DT)                                        \
   case DT:                                                   \
     status = launch_attention<DT, 1>(TLIE_ARGS);             \
@@ -772,7 +805,7 @@ static int attention_entry(const void* q, const void* cache, const int* block_ta
 #undef TLIE_ARGS
   if (status != kOk || nsplit == 1) return status;
   hipLaunchKernelGGL(attention_merge_kernel, dim3(tokens * nq), dim3(64), nsplit * sizeof(float), s, part_o, part_ml,
-                     (uint16_t*)out, nsplit, d, sink, nq);
+                     (uint16_t*)out, nsplit, d, sink, nq, (plane_map >> 24) & 1);
   return launch_status();
 }
 
@@ -785,6 +818,22 @@ extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* 
   // sink (or null): float [nq], a number per head whose exponential joins the softmax's denominator
   return attention_entry(q, cache, block_table, max_blocks, tiles, num_tiles, col_tiles, positions, out, part_o, part_ml, nsplit,
                          split_len, tokens, nq, nkv, d, page_size, window, chunk, sink, scale, waves, shared, stream);
+}
+
+// The same with planes of a page that several kv heads share (see the kernel's plane_map): key_share kv heads in a row
+// read one key plane (and q holds one query head for them), of every value_group kv heads in a row the i-th reads
+// value plane i % value_planes of the group's; float_out: out is float [tokens, nq, d].
+extern "C" int tlie_attention_mfma_planes(const void* q, const void* cache, const int* block_table, int max_blocks,
+                                          const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
+                                          float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
+                                          int d, int page_size, int window, int chunk, const float* sink, float scale, int waves,
+                                          int shared, int key_share, int value_group, int value_planes, int float_out,
+                                          void* stream) {
+  if (key_share <= 0 || key_share > 255 || value_group <= 0 || value_group > 255 || value_planes <= 0 || value_planes > 255)
+    return kBadArgument;
+  const int plane_map = key_share | (value_group << 8) | (value_planes << 16) | ((float_out ? 1 : 0) << 24);
+  return attention_entry(q, cache, block_table, max_blocks, tiles, num_tiles, col_tiles, positions, out, part_o, part_ml, nsplit,
+                         split_len, tokens, nq, nkv, d, page_size, window, chunk, sink, scale, waves, shared, stream, plane_map);
 }
 
 // ---- the same attention for callers that cannot allocate (declared and described in no_alloc.h) ----------

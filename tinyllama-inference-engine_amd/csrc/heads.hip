@@ -7,37 +7,41 @@
 //
 // Two maps: `a` then holds 2 * heads results a token in the order in which the attention kernel wants its
 // query heads, those of one key head side by side: with r = heads / (key/value groups), head h = g * r + i has
-// its first map at (2 g) * r + i and its second at (2 g + 1) * r + i.
+// its first map at (2 g) * r + i and its second at (2 g + 1) * r + i.  A map's result may also come in `parts`
+// pieces of dv / parts dims each (the attention kernel on the matrix cores takes value heads wider than the keys as
+// several heads of the keys' size): piece p of the map of key head k = 2 g + m lies at ((k * parts + p) * r + i).
 #include "common.h"
 
 namespace tlie {
 
 template <typename D, typename W, typename A>
 __global__ void __launch_bounds__(256)
-head_combine_kernel(const float* __restrict__ a, int heads, int dv, int pair_group, float lambda, float eps,
+head_combine_kernel(const float* __restrict__ a, int heads, int dv, int pair_group, int parts, float lambda, float eps,
                     const W* __restrict__ weight, float mult, const D* __restrict__ gate, int gate_nsplit,
                     size_t gate_split_stride, int gate_row, int gate_col, A* __restrict__ out) {
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int h = blockIdx.y * 4 + wave;
   if (h >= heads) return;                              // (a whole wave; no barrier follows)
-  const float* first;
-  const float* second = nullptr;
-  if (pair_group > 0) {
-    const int g = h / pair_group, i = h - g * pair_group;
-    const size_t row = static_cast<size_t>(t) * 2 * heads;
-    first = a + (row + static_cast<size_t>(2 * g) * pair_group + i) * dv;
-    second = a + (row + static_cast<size_t>(2 * g + 1) * pair_group + i) * dv;
-  } else {
-    first = a + (static_cast<size_t>(t) * heads + h) * dv;
-  }
+  // where dim e of the head's first (and second) result lies: with two maps, a map's result may come in `parts`
+  // pieces of dv / parts dims, the pieces of one key head's query heads piece by piece
+  const int piece = dv / parts;
+  const int g = pair_group > 0 ? h / pair_group : 0, i = pair_group > 0 ? h - g * pair_group : 0;
+  const float* row = a + static_cast<size_t>(t) * (pair_group > 0 ? 2 : 1) * heads * dv;
+  auto value = [&](int e) {
+    if (pair_group <= 0) return row[static_cast<size_t>(h) * dv + e];
+    const int p = e / piece, inside = e - p * piece;
+    const float first = row[((static_cast<size_t>(2 * g) * parts + p) * pair_group + i) * piece + inside];
+    const float second = row[((static_cast<size_t>(2 * g + 1) * parts + p) * pair_group + i) * piece + inside];
+    return first - lambda * second;
+  };
   float squares = 0.f;
   for (int e = lane; e < dv; e += 64) {
-    const float o = second != nullptr ? first[e] - lambda * second[e] : first[e];
+    const float o = value(e);
     squares += o * o;
   }
   const float r = 1.f / sqrtf(wave_sum(squares) / static_cast<float>(dv) + eps);
   for (int e = lane; e < dv; e += 64) {
-    const float o = second != nullptr ? first[e] - lambda * second[e] : first[e];
+    const float o = value(e);
     const int c = h * dv + e;
     float v = o * r * mult;
     if (weight != nullptr) v *= to_float(weight[c]);
@@ -55,18 +59,19 @@ using namespace tlie;
 
 // a: float [tokens, (pair_group > 0 ? 2 : 1) * heads, dv]; weight (or null): [heads * dv] of weight_dtype; gate (or null):
 // a product [nsplit][tokens][gate_row] of gate_dtype whose columns gate_col .. gate_col + heads * dv - 1 are read.
-extern "C" int tlie_head_combine(const float* a, int tokens, int heads, int dv, int pair_group, float lambda, float eps,
+extern "C" int tlie_head_combine(const float* a, int tokens, int heads, int dv, int pair_group, int parts, float lambda, float eps,
                                  const void* weight, int weight_dtype, float mult, const void* gate, int gate_dtype,
                                  int gate_nsplit, long long gate_split_stride, int gate_row, int gate_col, void* out,
                                  int out_dtype, void* stream) {
   if (tokens <= 0 || heads <= 0 || dv <= 0 || pair_group < 0 || (pair_group > 0 && heads % pair_group != 0)) return kBadArgument;
+  if (parts < 1 || dv % parts != 0 || (parts > 1 && pair_group <= 0)) return kBadArgument;
   if (gate != nullptr && (gate_nsplit < 1 || gate_col < 0 || gate_row < gate_col + heads * dv)) return kBadArgument;
   if (heads > 4 * 65535) return kBadArgument;
   const dim3 grid(tokens, (heads + 3) / 4);
   hipStream_t s = (hipStream_t)stream;
 #define TLIE_CASE(GC, D, WC, W, AC, A)                                                                                   \
   if (gate_dtype == GC && weight_dtype == WC && out_dtype == AC) {                                                       \
-    hipLaunchKernelGGL((head_combine_kernel<D, W, A>), grid, dim3(256), 0, s, a, heads, dv, pair_group, lambda, eps,      \
+    hipLaunchKernelGGL((head_combine_kernel<D, W, A>), grid, dim3(256), 0, s, a, heads, dv, pair_group, parts, lambda, eps,     \
                        (const W*)weight, mult, (const D*)gate, gate_nsplit, (size_t)gate_split_stride, gate_row, gate_col, \
                        (A*)out);                                                                                          \
     return launch_status();                                                                                              \

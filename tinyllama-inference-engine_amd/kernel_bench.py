@@ -340,3 +340,9 @@ def bench_design_kernels(sizes: dict, batch: int = 8, context: int = 2048, promp
             _timed(lambda i: ops.qkv_place(qkv, positions, slot_map, None, 0, cache, nq, nkv, d, d, bf), 4, samples),
             read_bytes=tokens * (nq + 2 * nkv) * d * 4)
     return rows
+
+
+def bench_raketar_kernels(sizes: dict, batch: int = 8, context: int = 2048, prompt: int = 2048, samples: int = 10, device="cuda:0",
+                          hbm_gbs: float = 8000.0, mfma_tflops: float = 2500.0) -> list[dict]:
+    """The kernels that the Raketar decoder adds, each alone at a layer's sizes (filled in below)."""
+    return []

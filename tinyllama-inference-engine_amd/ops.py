@@ -572,14 +572,18 @@ def gated_recurrence(fused: Product, x_col: int, y_col: int, u: torch.Tensor, ga
 
 def head_combine(a: torch.Tensor, heads: int, value_dim: int, eps: float, out_dtype: torch.dtype, pair_group: int = 0,
                  pair_lambda: float = 0.0, weight: torch.Tensor | None = None, mult: float = 1.0,
-                 gate: Product | None = None, gate_col: int = 0) -> torch.Tensor:
+                 gate: Product | None = None, gate_col: int = 0, parts: int = 1) -> torch.Tensor:
     """Each head's result normed by itself, on its way to the output product:
     out[t, h, :] = o / sqrt(mean(o^2) + eps) * weight[h] * mult * sigmoid(gate[t, h]), with o = a[t, h] or, for two maps
     of attention a head (pair_group > 0: the query heads of one key head lie side by side in `a`, pair_group of them,
     first all first maps' key heads ... see the kernel), o = first - pair_lambda * second.  a: float32
     [tokens, heads (or 2 * heads) * value_dim]; weight (or None): [heads * value_dim]; gate (or None): a product whose
-    columns gate_col .. gate_col + heads * value_dim hold the gate's pre-activations."""
+    columns gate_col .. gate_col + heads * value_dim hold the gate's pre-activations.  parts > 1 (with pair_group): a
+    map's result lies in `parts` pieces of value_dim / parts dims, each a head of its own of the attention kernel: the
+    pieces of a key head's query heads follow each other piece by piece (key head, piece, query head of the key head)."""
     _device_tensor(a, "a", torch.float32)
+    if parts < 1 or value_dim % parts != 0 or (parts > 1 and pair_group <= 0):
+        raise invalid_argument("head_combine: the pieces of a result must divide the value size (and go with two maps)")
     maps = 2 if pair_group > 0 else 1
     if a.dim() != 2 or a.shape[1] != maps * heads * value_dim:
         raise invalid_shape(f"head_combine: a {list(a.shape)} is not [tokens, {maps} * heads * value_dim]")
@@ -603,7 +607,7 @@ def head_combine(a: torch.Tensor, heads: int, value_dim: int, eps: float, out_dt
     out = torch.empty((tokens, heads * value_dim), dtype=out_dtype, device=a.device)
     if tokens == 0:
         return out
-    _check(library().tlie_head_combine(_ptr(a), tokens, heads, value_dim, pair_group, ctypes.c_float(pair_lambda),
+    _check(library().tlie_head_combine(_ptr(a), tokens, heads, value_dim, pair_group, int(parts), ctypes.c_float(pair_lambda),
                                        ctypes.c_float(eps), _ptr(weight), weight_code, ctypes.c_float(mult),
                                        _ptr(gate.data if gate is not None else None), gate_code, gate_nsplit,
                                        ctypes.c_longlong(gate_stride), gate_row, gate_col, _ptr(out), dtype_code(out_dtype),
@@ -1248,7 +1252,8 @@ def attention_mfma_takes(dtype: torch.dtype, head_dim: int, page_size: int) -> b
 def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor | None,
                    positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
                    scale: float, nsplit: int = 1, split_len: int = 0, col_tiles: int = 1, waves: int = 1,
-                   shared: bool = False, chunk: int | None = None, sink: torch.Tensor | None = None) -> torch.Tensor:
+                   shared: bool = False, chunk: int | None = None, sink: torch.Tensor | None = None,
+                   planes: tuple[int, int, int] | None = None, float_out: bool = False) -> torch.Tensor:
     """Causal attention of every token of the step over its sequence's cache, bfloat16.
 
     tiles: int32 [n, 4] from `attention_tiles` (built from the same step as block_table and
@@ -1262,8 +1267,21 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     with col_tiles * waves column groups, every wave takes col_tiles of them, and each block of keys
     and values is brought once for the whole workgroup.
     chunk: a token sees only the keys of its own chunk of so many positions (counted from position 0).
-    sink: float32 [nq], a number per head whose exponential joins the softmax's denominator."""
+    sink: float32 [nq], a number per head whose exponential joins the softmax's denominator.
+    planes (key_share, value_group, value_planes): kv heads share planes of a page: key_share kv heads in a row read
+    one key plane, and q holds one query head for them ([tokens, nq / key_share * d]); of every value_group kv heads in
+    a row the i-th reads value plane i % value_planes of that group's value_planes.  A page then holds
+    nkv / key_share planes of keys and after them nkv / value_group * value_planes planes of values, each
+    page_size * d (cache: [pages, ...] with so many values a page).  The result has all nq heads.
+    float_out (with planes): the result is float32."""
     _device_tensor(q, "q", torch.bfloat16)
+    if planes is not None:
+        key_share, value_group, value_planes = (int(v) for v in planes)
+        if (min(key_share, value_group, value_planes) <= 0 or max(key_share, value_group) > 255 or value_planes > value_group
+                or num_kv_heads % key_share != 0 or num_kv_heads % value_group != 0):
+            raise invalid_argument("attention: kv heads do not share planes that way")
+    elif float_out:
+        raise invalid_argument("attention: float results go with shared planes only")
     if sink is not None:
         _device_tensor(sink, "sink", torch.float32)
         if sink.shape != (num_heads,):
@@ -1274,9 +1292,20 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     _device_tensor(block_table, "block_table", torch.int32)
     _device_tensor(positions, "positions", torch.int32)
     tokens = q.shape[0]
-    if q.shape != (tokens, num_heads * head_dim):
-        raise invalid_shape(f"attention: q {list(q.shape)} is not [tokens, nq * d]")
-    page_size = _check_cache(cache, num_kv_heads, head_dim, "attention")
+    if num_kv_heads <= 0 or num_heads % num_kv_heads != 0:
+        raise invalid_shape("attention: the number of heads must be a multiple of the number of kv heads")
+    if planes is None:
+        if q.shape != (tokens, num_heads * head_dim):
+            raise invalid_shape(f"attention: q {list(q.shape)} is not [tokens, nq * d]")
+        page_size = _check_cache(cache, num_kv_heads, head_dim, "attention")
+    else:
+        if q.shape != (tokens, num_heads // key_share * head_dim):
+            raise invalid_shape(f"attention: q {list(q.shape)} is not [tokens, nq / key_share * d]")
+        per_row = (num_kv_heads // key_share + num_kv_heads // value_group * value_planes) * head_dim
+        per_page = cache[0].numel() if cache.dim() >= 2 and cache.shape[0] > 0 else 0
+        if per_page == 0 or per_page % per_row != 0:
+            raise invalid_shape(f"attention: cache {list(cache.shape)} does not hold pages of {per_row} values a position")
+        page_size = per_page // per_row
     if block_table.dim() != 2 or positions.shape != (tokens,):
         raise invalid_shape("attention: block_table must be [sequences, max_blocks], positions [tokens]")
     if num_heads % num_kv_heads != 0:
@@ -1304,11 +1333,19 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
         raise invalid_argument(f"attention: waves must be a power of two up to {attention_max_waves(head_dim, col_tiles)}")
     if not attention_mfma_takes(q.dtype, head_dim, page_size):
         raise invalid_argument("attention_mfma takes bfloat16, head sizes in steps of 16 up to 256, pages of a power of two of rows (at least 16)")
-    out = torch.empty_like(q)
+    out = torch.empty((tokens, num_heads * head_dim), dtype=torch.float32 if float_out else torch.bfloat16, device=q.device)
     part_o = part_ml = None
     if nsplit > 1:
         part_o = torch.empty((tokens * num_heads * nsplit, head_dim), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((tokens * num_heads * nsplit, 2), dtype=torch.float32, device=q.device)
+    if planes is not None:
+        _check(library().tlie_attention_mfma_planes(_ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(tiles),
+                                                    num_tiles, col_tiles, _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml),
+                                                    nsplit, split_len, tokens, num_heads, num_kv_heads, head_dim, page_size,
+                                                    int(window) if window else 0, int(chunk) if chunk else 0, _ptr(sink),
+                                                    ctypes.c_float(scale), waves, int(bool(shared)), key_share, value_group,
+                                                    value_planes, 1 if float_out else 0, _stream()), "attention_mfma")
+        return out
     _check(library().tlie_attention_mfma(_ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(tiles),
                                          num_tiles, col_tiles, _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), nsplit,
                                          split_len, tokens, num_heads, num_kv_heads, head_dim, page_size,

@@ -13,7 +13,9 @@ The two maps are two heads of an ordinary attention whose key heads come in pair
 layer runs as an attention of 2 * heads query heads over 2 * groups key heads and `groups` value heads, through
 the attention kernel, and a kernel of its own forms the difference, the norm and the gate.  Its results leave the
 attention kernel as floats, because their difference is normed.  A page of the cache holds the 2 * groups
-planes of keys [row][dim] and after them the `groups` planes of values, transposed, [dim][row].  The four
+planes of keys [row][dim] and after them the `groups` planes of values, transposed, [dim][row].  In bfloat16,
+with values a multiple of the keys' size, the kernel on the matrix cores reads the same pages: it takes a value
+head as so many pieces of the keys' size, each a head of its own whose scores are those of its map.  The four
 projections (q, k, v and the gate) are one product.
 """
 from __future__ import annotations
@@ -132,10 +134,22 @@ class DifferentialAttention(Mixer):
         q = ops.qkv_place(fused, ctx.positions, pages.slot_map if binding.writes else ctx.no_slots, inv_freq, rot_dim,
                           binding.cache, heads, key_heads, self.d, self.dv, self.dtype, value_heads=self.groups,
                           extra_cols=gate_cols)
-        attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, heads, key_heads,
-                                         self.d, None, self.scale, tiled=ops.attention_generic_plan(ctx, self.d, self.dv),
-                                         seq_start=ctx.seq_start, value_dim=self.dv, value_heads=self.groups, float_out=True)
+        page_size = binding.cache.shape[2] // (2 * self.d + self.dv)
+        parts = 1
+        if self.dv % self.d == 0 and self.dv // self.d <= 64 and ops.attention_mfma_takes(self.dtype, self.d, page_size):
+            # bfloat16, values a multiple of the keys' size: the kernel on the matrix cores.  A value head's pieces of
+            # the keys' size are kv heads of that kernel: key head k and piece p make kv head k * parts + p, which reads
+            # key plane k and, with its map's partner, the group's value planes
+            parts = self.dv // self.d
+            tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, self.per_group, key_heads * parts, self.d)
+            attended = ops.attention_mfma(q, binding.cache, pages.block_table, tiles, ctx.positions, heads * parts, key_heads * parts,
+                                          self.d, None, self.scale, nsplit, split_len, col_tiles, waves, shared,
+                                          planes=(parts, 2 * parts, parts), float_out=True)
+        else:
+            attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, heads, key_heads,
+                                             self.d, None, self.scale, tiled=ops.attention_generic_plan(ctx, self.d, self.dv),
+                                             seq_start=ctx.seq_start, value_dim=self.dv, value_heads=self.groups, float_out=True)
         combined = ops.head_combine(attended, self.heads, self.dv, self.eps, self.dtype, pair_group=self.per_group,
                                     pair_lambda=self.pair_lambda, mult=1.0 - self.diff,
-                                    gate=fused if self.output_gate else None, gate_col=fused.cols - gate_cols)
+                                    gate=fused if self.output_gate else None, gate_col=fused.cols - gate_cols, parts=parts)
         return self.o(combined)
