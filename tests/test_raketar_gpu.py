@@ -145,29 +145,33 @@ def test_routed_gate_scales_an_experts_columns(tokens, experts, block, shared, n
     assert float((got.cpu().double() - want).abs().max()) < 2e-5
 
 
-@pytest.mark.parametrize("tokens,width,side_dim,nsplit,second", [(6, 96, 10, 1, True), (3, 200, 3, 2, True), (20, 64, 24, 1, False)])
-def test_residual_update_with_and_without_a_token_input(tokens, width, side_dim, nsplit, second):
+@pytest.mark.parametrize("tokens,width,nsplit,second", [(6, 96, 1, True), (3, 200, 2, True), (20, 64, 1, False)])
+def test_residual_update_adds_both_results_and_leaves_a_copy(tokens, width, nsplit, second):
     from tlie_amd import ops
     generator = torch.Generator().manual_seed(width)
-    vocab, layers, layer, mult, eps = 30, 3, 1, 0.45, 1e-5
+    mult = 0.45
     x, a, b = (torch.randn(tokens, width, generator=generator) for _ in range(3))
-    ids = torch.randint(0, vocab, (tokens,), generator=generator)
-    table = torch.randn(vocab, layers * side_dim, generator=generator)
-    gate, proj = torch.randn(side_dim, width, generator=generator) * 0.2, torch.randn(width, side_dim, generator=generator)
-    norm = torch.randn(width, generator=generator)
     summed = x.double() + mult * (a.double() + (b.double() if second else 0.0))
     residual = x.clone().to(DEVICE)
-    ops.residual_update(residual, split_product(a, nsplit, generator), split_product(b, nsplit, generator) if second else None, mult)
+    assert ops.residual_update(residual, split_product(a, nsplit, generator), split_product(b, nsplit, generator) if second else None, mult) is None
     assert float((residual.cpu().double() - summed).abs().max()) < 1e-5
-    config = {"token_side": {"dim": side_dim}}
-    w = {"side.embed": table.double(), f"l{layer}.side.gate": gate.double(), f"l{layer}.side.proj": proj.double(),
-         f"l{layer}.side.norm": norm.double()}
-    want = plain.token_side(config, w, layer, ids, summed, mult, eps)
     residual = x.clone().to(DEVICE)
-    side = ops.SideInput(table.to(DEVICE), layer * side_dim, side_dim, gate.to(DEVICE), proj.to(DEVICE), norm.to(DEVICE), eps)
-    ops.residual_update(residual, split_product(a, nsplit, generator), split_product(b, nsplit, generator) if second else None, mult,
-                        side=side, tokens=ids.to(torch.int32).to(DEVICE))
-    assert float((residual.cpu().double() - want).abs().max()) < 3e-5
+    copy = ops.residual_update(residual, split_product(a, nsplit, generator), split_product(b, nsplit, generator) if second else None, mult,
+                               copy_dtype=torch.bfloat16)
+    assert copy.dtype == torch.bfloat16 and torch.equal(copy, residual.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("tokens,side_dim,nsplit", [(6, 10, 1), (3, 3, 2), (20, 24, 1)])
+def test_the_token_inputs_gate(tokens, side_dim, nsplit):
+    from tlie_amd import ops
+    generator = torch.Generator().manual_seed(side_dim)
+    vocab, layers, layer = 30, 3, 1
+    pre = torch.randn(tokens, side_dim, generator=generator) * 2.0
+    ids = torch.randint(0, vocab, (tokens,), generator=generator)
+    table = torch.randn(vocab, layers * side_dim, generator=generator)
+    want = plain.gelu_tanh(pre.double()) * table.double()[ids][:, layer * side_dim:(layer + 1) * side_dim]
+    got = ops.side_gate(split_product(pre, nsplit, generator), ids.to(torch.int32).to(DEVICE), table.to(DEVICE), layer * side_dim, torch.float32)
+    assert float((got.cpu().double() - want).abs().max()) < 1e-5
 
 
 def test_residual_inject_adds_the_embedding_and_a_vector():
@@ -425,7 +429,7 @@ def test_every_layer_matches_the_plain_implementation(setups, name):
     engine.step([StepEntry("a", tokens, [len(tokens) - 1])], trace=trace)
     assert len(layers) == len(engine.spec.runs)
     for index, want in enumerate(layers):
-        assert_rows(trace[f"layer{index}.output"], want, 1e-5, f"{name}: the residual after run {index}")
+        assert_rows(trace[f"layer{index}.output"], want, TOLERANCE["float32"], f"{name}: the residual after run {index}")
 
 
 @pytest.mark.parametrize("name,dtype", CASES)

@@ -9,53 +9,110 @@
 // S, n and m are the request's state (zero when it is admitted) and are carried from step to step; all of
 // this is float whatever type q, k and v come in.
 //
-// A workgroup is one wave and owns 64 columns of one head's S for one sequence of the step: lane l keeps
-// column l of its tile, S[0 .. dim)[l], in registers, and walks the sequence's tokens of the step in order.
-// n is spread over the lanes (lane l keeps n[l], n[l + 64], ...), every tile keeps a copy of its own of n
-// and m (so that no workgroup reads what another one writes), and the state row of a head is laid out tile
-// by tile: [tiles][dim * 64 (S, [d][lane]) + dim (n) + 1 (m)].  Queries and keys of four tokens at a time go
-// through LDS (every lane needs all of them); the order of a token's sums never depends on how the step
-// was cut or on what else is in it.
+// The gates do not depend on the memory: a first kernel walks each sequence's gates alone and leaves, per token and
+// head, keep = exp(f + m - m'), take = exp(i - m') and exp(-m'), and the head's m after the step in the state.
+//
+// The memory itself: a workgroup is one wave and owns 64 columns of one head's S for one sequence of the step: lane l
+// keeps column l of its tile, S[0 .. dim)[l], in registers, and walks tokens in order.  n is spread over the lanes
+// (lane l keeps n[l], n[l + 64], ...), every tile keeps a copy of its own of n (so that no workgroup reads what
+// another one writes), and the state row of a head is laid out tile by tile:
+// [tiles][dim * 64 (S, [d][lane]) + dim (n) + 1 (m, the first tile's only)].  Queries and keys of four tokens at a time
+// go through LDS (every lane needs all of them).
+//
+// A sequence that brings many tokens is taken in slices of 64 tokens that run side by side: every slice is walked
+// from a memory of zero and leaves where it ends and the product of its keeps (S' = keep S + take k v^T is linear
+// in S); a second kernel gives every slice its start, start(c + 1) = keeps(c) * start(c) + end(c), and the state its
+// new value; a third walks every slice again from its start and writes the results.
 #include "common.h"
 
 namespace tlie {
 
-constexpr int kMlstmBatch = 4;
+constexpr int kMlstmBatch = 4, kMlstmSlice = 64;
 
-template <typename D, int DMAX>
+// gates: float [tokens, 2 * heads] (input gates' pre-activations, then forget gates'); values: float [tokens, heads, 4]
+// (keep, take, exp(-m), unused).  One wave per (sequence, head); m is the state's, read and written here only.
+__global__ void __launch_bounds__(64)
+mlstm_gates_kernel(const float* __restrict__ gates, float* __restrict__ values, float* __restrict__ state,
+                   const int* __restrict__ seq_start, const int* __restrict__ seq_slot, int heads, size_t head_floats,
+                   size_t m_offset, float cap) {
+  __shared__ float log_i[64], log_f[64], maxima[65];
+  const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int slot = seq_slot[seq];
+  if (slot < 0) return;
+  const int first = seq_start[seq], last = seq_start[seq + 1];
+  if (first >= last) return;
+  float* m_place = state + (static_cast<size_t>(slot) * heads + h) * head_floats + m_offset;
+  float m = *m_place;
+  for (int t0 = first; t0 < last; t0 += 64) {
+    const int t = t0 + lane, count = min(64, last - t0);
+    float ig = 0.f, fg = 0.f;
+    if (lane < count) {
+      ig = cap * tanhf(gates[static_cast<size_t>(t) * 2 * heads + h] / cap);
+      const float x = cap * tanhf(gates[static_cast<size_t>(t) * 2 * heads + heads + h] / cap);
+      fg = fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
+    }
+    __syncthreads();
+    log_i[lane] = ig, log_f[lane] = fg;
+    __syncthreads();
+    if (lane == 0) {                                   // the running maximum, token by token
+      maxima[0] = m;
+      for (int j = 0; j < count; ++j) maxima[j + 1] = fmaxf(log_f[j] + maxima[j], log_i[j]);
+    }
+    __syncthreads();
+    if (lane < count) {
+      const float before = maxima[lane], after = maxima[lane + 1];
+      float4 out;
+      out.x = expf(fg + before - after), out.y = expf(ig - after), out.z = expf(-after), out.w = 0.f;
+      *reinterpret_cast<float4*>(values + (static_cast<size_t>(t) * heads + h) * 4) = out;
+    }
+    m = maxima[count];
+  }
+  if (lane == 0) *m_place = m;
+}
+
+// MODE 0: the sequence's tokens of the step from the state, results and the new state written.
+// MODE 1: a slice from zero; no results; where it ends and the product of its keeps go to `parts`.
+// MODE 2: a slice from the start that `parts` now holds for it; results written.
+// parts: float [sequences, slices, heads, tiles, dim * 64 + dim + 1] (S, n, the product of the slice's keeps).
+template <typename D, int DMAX, int MODE>
 __global__ void __launch_bounds__(64)
 mlstm_scan_kernel(const D* __restrict__ fused, int nsplit, size_t split_stride, int row_width, int q_col, int k_col,
-                  int v_col, const float* __restrict__ gates, float* __restrict__ state,
+                  int v_col, const float* __restrict__ values, float* __restrict__ state, float* __restrict__ parts,
                   const int* __restrict__ seq_start, const int* __restrict__ seq_slot, float* __restrict__ out, int heads,
-                  int dim, int vdim, int tiles, float cap, float q_scale) {
+                  int dim, int vdim, int tiles, int slices, float q_scale) {
   constexpr int NJ = DMAX >= 64 ? DMAX / 64 : 1;
   __shared__ __attribute__((aligned(16))) float qs[kMlstmBatch][DMAX];
   __shared__ __attribute__((aligned(16))) float ks[kMlstmBatch][DMAX];
-  const int seq = blockIdx.x, h = blockIdx.y, tile = blockIdx.z, lane = threadIdx.x;
+  const int seq = MODE == 0 ? blockIdx.x : blockIdx.x / slices, slice = MODE == 0 ? 0 : blockIdx.x % slices;
+  const int h = blockIdx.y, tile = blockIdx.z, lane = threadIdx.x;
   const int slot = seq_slot[seq];
   if (slot < 0) return;                                // a sequence that pads a recorded step: no state is its own
-  const int first = seq_start[seq], last = seq_start[seq + 1];
+  int first = seq_start[seq], last = seq_start[seq + 1];
+  if (MODE != 0) {
+    first += slice * kMlstmSlice;
+    last = min(last, first + kMlstmSlice);
+  }
   if (first >= last) return;
   const int col = tile * 64 + lane;
   const bool live = col < vdim;
   const size_t tile_floats = static_cast<size_t>(dim) * 64 + dim + 1;
-  float* st = state + ((static_cast<size_t>(slot) * heads + h) * tiles + tile) * tile_floats;
+  float* st = MODE == 0 ? state + ((static_cast<size_t>(slot) * heads + h) * tiles + tile) * tile_floats
+                        : parts + (((static_cast<size_t>(seq) * slices + slice) * heads + h) * tiles + tile) * tile_floats;
   float S[DMAX];
-#pragma unroll
-  for (int d = 0; d < DMAX; ++d) S[d] = d < dim ? st[d * 64 + lane] : 0.f;
   float n[NJ];
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d) S[d] = MODE != 1 && d < dim ? st[d * 64 + lane] : 0.f;
 #pragma unroll
   for (int j = 0; j < NJ; ++j) {
     const int d = lane + 64 * j;
-    n[j] = d < dim ? st[static_cast<size_t>(dim) * 64 + d] : 0.f;
+    n[j] = MODE != 1 && d < dim ? st[static_cast<size_t>(dim) * 64 + d] : 0.f;
   }
-  float m = st[static_cast<size_t>(dim) * 64 + dim];
-  const int gate_row = 2 * heads;
+  float keeps = 1.f;
 
   for (int t0 = first; t0 < last; t0 += kMlstmBatch) {
     const int nb = min(kMlstmBatch, last - t0);
     __syncthreads();                                   // the batch before has been read
-    float vv[kMlstmBatch], gi[kMlstmBatch], gf[kMlstmBatch];
+    float vv[kMlstmBatch], keep[kMlstmBatch], take[kMlstmBatch], floor_[kMlstmBatch];
 #pragma unroll
     for (int b = 0; b < kMlstmBatch; ++b) {
       const D* row = fused + static_cast<size_t>(t0 + b) * row_width;
@@ -64,39 +121,36 @@ mlstm_scan_kernel(const D* __restrict__ fused, int nsplit, size_t split_stride, 
         const int d = lane + 64 * j;
         if (d < DMAX) {
           const bool there = b < nb && d < dim;
-          qs[b][d] = there ? sum_splits(row + q_col + h * dim + d, nsplit, split_stride) * q_scale : 0.f;
+          if (MODE != 1) qs[b][d] = there ? sum_splits(row + q_col + h * dim + d, nsplit, split_stride) * q_scale : 0.f;
           ks[b][d] = there ? sum_splits(row + k_col + h * dim + d, nsplit, split_stride) : 0.f;
         }
       }
       vv[b] = b < nb && live ? sum_splits(row + v_col + h * vdim + col, nsplit, split_stride) : 0.f;
-      gi[b] = b < nb ? gates[static_cast<size_t>(t0 + b) * gate_row + h] : 0.f;
-      gf[b] = b < nb ? gates[static_cast<size_t>(t0 + b) * gate_row + heads + h] : 0.f;
+      const float4 gate = b < nb ? *reinterpret_cast<const float4*>(values + (static_cast<size_t>(t0 + b) * heads + h) * 4)
+                                 : make_float4(1.f, 0.f, 1.f, 0.f);
+      keep[b] = gate.x, take[b] = gate.y, floor_[b] = gate.z;
     }
     __syncthreads();
 #pragma unroll
     for (int b = 0; b < kMlstmBatch; ++b) {
       if (b >= nb) break;                              // (the same for the whole wave)
-      const float ig = cap * tanhf(gi[b] / cap);
-      const float x = cap * tanhf(gf[b] / cap);
-      const float fg = fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
-      const float m_new = fmaxf(fg + m, ig);
-      const float keep = expf(fg + m - m_new), take = expf(ig - m_new);
-      m = m_new;
-      const float tv = take * vv[b];
+      const float tv = take[b] * vv[b];
       float acc = 0.f;
 #pragma unroll
       for (int d0 = 0; d0 < DMAX; d0 += 4) {
         if (d0 < dim) {                                // (entries from dim on are zeros in LDS and stay zeros in S)
           const float4 k4 = *reinterpret_cast<const float4*>(&ks[b][d0]);
-          const float4 q4 = *reinterpret_cast<const float4*>(&qs[b][d0]);
-          S[d0 + 0] = keep * S[d0 + 0] + k4.x * tv;
-          acc += S[d0 + 0] * q4.x;
-          S[d0 + 1] = keep * S[d0 + 1] + k4.y * tv;
-          acc += S[d0 + 1] * q4.y;
-          S[d0 + 2] = keep * S[d0 + 2] + k4.z * tv;
-          acc += S[d0 + 2] * q4.z;
-          S[d0 + 3] = keep * S[d0 + 3] + k4.w * tv;
-          acc += S[d0 + 3] * q4.w;
+          S[d0 + 0] = keep[b] * S[d0 + 0] + k4.x * tv;
+          S[d0 + 1] = keep[b] * S[d0 + 1] + k4.y * tv;
+          S[d0 + 2] = keep[b] * S[d0 + 2] + k4.z * tv;
+          S[d0 + 3] = keep[b] * S[d0 + 3] + k4.w * tv;
+          if (MODE != 1) {
+            const float4 q4 = *reinterpret_cast<const float4*>(&qs[b][d0]);
+            acc += S[d0 + 0] * q4.x;
+            acc += S[d0 + 1] * q4.y;
+            acc += S[d0 + 2] * q4.z;
+            acc += S[d0 + 3] * q4.w;
+          }
         }
       }
       float partial = 0.f;
@@ -104,15 +158,20 @@ mlstm_scan_kernel(const D* __restrict__ fused, int nsplit, size_t split_stride, 
       for (int j = 0; j < NJ; ++j) {
         const int d = lane + 64 * j;
         if (d < DMAX) {
-          n[j] = keep * n[j] + take * ks[b][d];
-          partial += n[j] * qs[b][d];
+          n[j] = keep[b] * n[j] + take[b] * ks[b][d];
+          if (MODE != 1) partial += n[j] * qs[b][d];
         }
       }
-      const float nq = wave_sum(partial);
-      const float bottom = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
-      if (live) out[(static_cast<size_t>(t0 + b) * heads + h) * vdim + col] = acc / bottom;
+      if (MODE == 1) {
+        keeps *= keep[b];
+      } else {
+        const float nq = wave_sum(partial);
+        const float bottom = fmaxf(fabsf(nq), floor_[b]) + 1e-6f;
+        if (live) out[(static_cast<size_t>(t0 + b) * heads + h) * vdim + col] = acc / bottom;
+      }
     }
   }
+  if (MODE == 2) return;
 #pragma unroll
   for (int d = 0; d < DMAX; ++d)
     if (d < dim) st[d * 64 + lane] = S[d];
@@ -121,7 +180,32 @@ mlstm_scan_kernel(const D* __restrict__ fused, int nsplit, size_t split_stride, 
     const int d = lane + 64 * j;
     if (d < dim) st[static_cast<size_t>(dim) * 64 + d] = n[j];
   }
-  if (lane == 0) st[static_cast<size_t>(dim) * 64 + dim] = m;
+  if (MODE == 1 && lane == 0) st[static_cast<size_t>(dim) * 64 + dim] = keeps;
+}
+
+// Every slice's start from the state and the slices before it, in place: where a slice's end stood its start stands
+// afterwards; the state gets what the last slice leaves.  A thread an element of (S, n) of a (sequence, head, tile).
+__global__ void __launch_bounds__(256)
+mlstm_carry_kernel(float* __restrict__ parts, float* __restrict__ state, const int* __restrict__ seq_start,
+                   const int* __restrict__ seq_slot, int heads, int tiles, int slices, int dim) {
+  const int seq = blockIdx.x, unit = blockIdx.y;       // unit: head * tiles + tile
+  const int slot = seq_slot[seq];
+  if (slot < 0) return;
+  const int count = seq_start[seq + 1] - seq_start[seq];
+  const int used = (count + kMlstmSlice - 1) / kMlstmSlice;
+  const size_t tile_floats = static_cast<size_t>(dim) * 64 + dim + 1;
+  const int elements = dim * 64 + dim;
+  float* st = state + (static_cast<size_t>(slot) * heads * tiles + unit) * tile_floats;
+  for (int e = blockIdx.z * 256 + threadIdx.x; e < elements; e += gridDim.z * 256) {
+    float value = st[e];
+    for (int c = 0; c < used; ++c) {
+      float* part = parts + ((static_cast<size_t>(seq) * slices + c) * heads * tiles + unit) * tile_floats;
+      const float end = part[e], keeps = part[elements];
+      part[e] = value;
+      value = keeps * value + end;
+    }
+    if (used > 0) st[e] = value;
+  }
 }
 
 }  // namespace tlie
@@ -130,30 +214,55 @@ using namespace tlie;
 
 // fused: a product [nsplit][tokens][row_width] whose columns q_col .. hold the heads' queries (dim each), k_col ..
 // their keys, v_col .. their values (vdim each); gates: float [tokens, 2 * heads], the input gates' and then the
-// forget gates' pre-activations; state: float [slots, heads, tiles, dim * 64 + dim + 1], tiles = ceil(vdim / 64);
-// seq_start [sequences + 1], seq_slot [sequences] (negative: skipped); out: float [tokens, heads * vdim].
+// forget gates' pre-activations; values: float [tokens, heads, 4], scratch for what the gates become; state: float
+// [slots, heads, tiles, dim * 64 + dim + 1], tiles = ceil(vdim / 64); seq_start [sequences + 1], seq_slot [sequences]
+// (negative: skipped); out: float [tokens, heads * vdim].  slices 0: every sequence's tokens are walked in order;
+// slices > 0 (at least ceil(most tokens of a sequence / 64)): in slices of 64 tokens side by side, with parts: float
+// [sequences, slices, heads, tiles, dim * 64 + dim + 1] as scratch.
 extern "C" int tlie_mlstm_scan(const void* fused, int dtype, int nsplit, long long split_stride, int row_width, int q_col,
-                               int k_col, int v_col, const float* gates, float* state, const int* seq_start,
+                               int k_col, int v_col, const float* gates, float* values, float* state, const int* seq_start,
                                const int* seq_slot, float* out, int sequences, int heads, int dim, int vdim, float cap,
-                               float q_scale, void* stream) {
+                               float q_scale, int slices, float* parts, void* stream) {
   if (sequences <= 0 || heads <= 0 || dim <= 0 || dim > 256 || vdim <= 0 || nsplit < 1 || !(cap > 0.f)) return kBadArgument;
   const int tiles = (vdim + 63) / 64;
-  if (heads > 65535 || tiles > 65535) return kBadArgument;
+  if (heads > 65535 || tiles > 65535 || slices < 0 || (slices > 0 && parts == nullptr) || values == nullptr) return kBadArgument;
   if (q_col < 0 || k_col < 0 || v_col < 0 || q_col + heads * dim > row_width || k_col + heads * dim > row_width ||
       v_col + heads * vdim > row_width)
     return kBadArgument;
-  const dim3 grid(sequences, heads, tiles);
   hipStream_t s = (hipStream_t)stream;
-#define TLIE_LAUNCH(D, DMAX)                                                                                          \
-  hipLaunchKernelGGL((mlstm_scan_kernel<D, DMAX>), grid, dim3(64), 0, s, (const D*)fused, nsplit, (size_t)split_stride, \
-                     row_width, q_col, k_col, v_col, gates, state, seq_start, seq_slot, out, heads, dim, vdim, tiles,  \
-                     cap, q_scale)
-#define TLIE_SIZES(D)                                                                                                 \
-  if (dim <= 32) TLIE_LAUNCH(D, 32); else if (dim <= 64) TLIE_LAUNCH(D, 64); else if (dim <= 128) TLIE_LAUNCH(D, 128); \
-  else TLIE_LAUNCH(D, 256)
-  if (dtype == kF32) { TLIE_SIZES(float); }
-  else if (dtype == kBF16) { TLIE_SIZES(bf16); }
-  else return kBadArgument;
+  const size_t tile_floats = static_cast<size_t>(dim) * 64 + dim + 1;
+  hipLaunchKernelGGL(mlstm_gates_kernel, dim3(sequences, heads), dim3(64), 0, s, gates, values, state, seq_start, seq_slot,
+                     heads, tiles * tile_floats, tile_floats - 1, cap);
+  if (launch_status() != kOk) return kLaunchFailed;
+#define TLIE_LAUNCH(D, DMAX, MODE, GRID)                                                                              \
+  hipLaunchKernelGGL((mlstm_scan_kernel<D, DMAX, MODE>), GRID, dim3(64), 0, s, (const D*)fused, nsplit,                \
+                     (size_t)split_stride, row_width, q_col, k_col, v_col, values, state, parts, seq_start, seq_slot,  \
+                     out, heads, dim, vdim, tiles, slices, q_scale)
+#define TLIE_SIZES(D, MODE, GRID)                                                                                     \
+  if (dim <= 32) TLIE_LAUNCH(D, 32, MODE, GRID); else if (dim <= 64) TLIE_LAUNCH(D, 64, MODE, GRID);                  \
+  else if (dim <= 128) TLIE_LAUNCH(D, 128, MODE, GRID); else TLIE_LAUNCH(D, 256, MODE, GRID)
+#define TLIE_TYPES(MODE, GRID)                                                                                        \
+  if (dtype == kF32) { TLIE_SIZES(float, MODE, GRID); }                                                               \
+  else if (dtype == kBF16) { TLIE_SIZES(bf16, MODE, GRID); }                                                          \
+  else return kBadArgument
+  if (slices == 0) {
+    const dim3 grid(sequences, heads, tiles);
+    TLIE_TYPES(0, grid);
+    return launch_status();
+  }
+  if (static_cast<long long>(sequences) * slices > 2147483647LL) return kBadArgument;
+  const dim3 sliced(sequences * slices, heads, tiles);
+  TLIE_TYPES(1, sliced);
+  if (launch_status() != kOk) return kLaunchFailed;
+  const int elements = dim * 64 + dim;
+  int across = (elements + 255) / 256;
+  if (across > 16) across = 16;
+  if (heads * tiles > 65535) return kBadArgument;
+  hipLaunchKernelGGL(mlstm_carry_kernel, dim3(sequences, heads * tiles, across), dim3(256), 0, s, parts, state, seq_start,
+                     seq_slot, heads, tiles, slices, dim);
+  if (launch_status() != kOk) return kLaunchFailed;
+  TLIE_TYPES(2, sliced);
+#undef TLIE_TYPES
 #undef TLIE_SIZES
 #undef TLIE_LAUNCH
   return launch_status();

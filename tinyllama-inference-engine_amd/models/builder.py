@@ -106,7 +106,7 @@ class DecoderModel:
             if run.add_embedding or run.add_vector is not None:
                 # what a run takes in before it starts: the residual is brought up to date first
                 if pending is not None and not isinstance(pending, ResidualUpdated):
-                    self._settle(residual, pending)
+                    self._settle(residual, pending, self.dtype)
                     pending = None
                 vector = self.run_vectors[run.add_vector[0]][run.add_vector[1]] if run.add_vector is not None else None
                 ops.residual_inject(residual, ctx.tokens, self.embedding.table if run.add_embedding else None, vector)
@@ -127,10 +127,10 @@ class DecoderModel:
 
 
     @staticmethod
-    def _settle(residual, pending) -> None:
+    def _settle(residual, pending, dtype) -> None:
         """Adds what a block handed on into the residual now (a block whose result waits for the next norm)."""
         if isinstance(pending, ops.NormedDelta):
-            ops.norm_add_rmsnorm(residual, pending.product, pending.weight, pending.eps, None, pending.eps, residual.dtype)
+            ops.norm_add_rmsnorm(residual, pending.product, pending.weight, pending.eps, None, pending.eps, dtype)
         else:
             residual += ops.as_product(pending).dense(torch.float32)
 

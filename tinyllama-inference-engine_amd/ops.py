@@ -616,6 +616,8 @@ def head_combine(a: torch.Tensor, heads: int, value_dim: int, eps: float, out_dt
 
 
 MLSTM_MAX_DIM = 256            # the largest query/key size of a head that the matrix-memory kernel keeps in registers
+MLSTM_SLICE = 64               # tokens of a slice of the sliced walk (the kernel's kMlstmSlice)
+MLSTM_SLICED_FROM = 192        # tokens a sequence brings from which the sliced walk pays (two walks of a slice and a carry)
 
 
 def mlstm_state_shape(heads: int, dim: int, value_dim: int) -> tuple[int, ...]:
@@ -625,11 +627,14 @@ def mlstm_state_shape(heads: int, dim: int, value_dim: int) -> tuple[int, ...]:
 
 def mlstm_scan(fused: Product, q_col: int, k_col: int, v_col: int, gates: torch.Tensor, state: torch.Tensor,
                seq_start: torch.Tensor, seq_slot: torch.Tensor, heads: int, dim: int, value_dim: int, cap: float,
-               q_scale: float) -> torch.Tensor:
+               q_scale: float, max_new: int = 1) -> torch.Tensor:
     """The matrix memory of an mLSTM layer over the step's tokens, sequence by sequence (see csrc/mlstm.hip): reads
     q, k, v from the product's columns, the gates' pre-activations from `gates` (float32 [tokens, 2 * heads]: input
     gates, then forget gates), carries `state` (float32 [slots, *mlstm_state_shape]) for sequences whose slot is not
-    negative, and returns float32 [tokens, heads * value_dim], the heads' results before their norm."""
+    negative, and returns float32 [tokens, heads * value_dim], the heads' results before their norm.  max_new: the
+    most tokens any sequence brings in this step (the caller knows it on the host); from MLSTM_SLICED_FROM on the
+    sequences' tokens are taken in slices of MLSTM_SLICE that run side by side, each from the start that the slices
+    before it leave; else every sequence's tokens are walked in order."""
     _check_product(fused, "fused")
     _device_tensor(gates, "gates", torch.float32)
     _device_tensor(state, "state", torch.float32)
@@ -651,10 +656,16 @@ def mlstm_scan(fused: Product, q_col: int, k_col: int, v_col: int, gates: torch.
     out = torch.empty((tokens, heads * value_dim), dtype=torch.float32, device=state.device)
     if tokens == 0 or sequences == 0:
         return out
+    values = torch.empty((tokens, heads, 4), dtype=torch.float32, device=state.device)
+    slices, parts = 0, None
+    if max_new >= MLSTM_SLICED_FROM:
+        slices = (min(int(max_new), tokens) + MLSTM_SLICE - 1) // MLSTM_SLICE
+        parts = torch.empty((sequences, slices, *state.shape[1:]), dtype=torch.float32, device=state.device)
     _check(library().tlie_mlstm_scan(_ptr(fused.data), dtype_code(fused.data.dtype), fused.nsplit,
                                      ctypes.c_longlong(fused.split_stride), fused.cols, q_col, k_col, v_col, _ptr(gates),
-                                     _ptr(state), _ptr(seq_start), _ptr(seq_slot), _ptr(out), sequences, heads, dim,
-                                     value_dim, ctypes.c_float(cap), ctypes.c_float(q_scale), _stream()), "mlstm_scan")
+                                     _ptr(values), _ptr(state), _ptr(seq_start), _ptr(seq_slot), _ptr(out), sequences, heads,
+                                     dim, value_dim, ctypes.c_float(cap), ctypes.c_float(q_scale), slices, _ptr(parts),
+                                     _stream()), "mlstm_scan")
     return out
 
 
@@ -702,57 +713,45 @@ def routed_gate(gate_up: Product, scale: torch.Tensor, block: int, out_dtype: to
     return out
 
 
-@dataclass
-class SideInput:
-    """A per-layer token input for `residual_update`: the table [vocab, row] of which columns offset .. offset + dim
-    are the layer's, the gate [dim, width], the projection [width, dim], the norm's weight [width] and its eps."""
-    table: torch.Tensor
-    offset: int
-    dim: int
-    gate: torch.Tensor
-    proj: torch.Tensor
-    norm: torch.Tensor
-    eps: float
-
-
-RESIDUAL_UPDATE_MAX_WIDTH = 8000       # with a side input the kernel keeps two rows of floats in LDS
-
-
 def residual_update(residual: torch.Tensor, first: Product, second: Product | None, mult: float,
-                    side: SideInput | None = None, tokens: torch.Tensor | None = None) -> None:
-    """residual += mult * (first + second), in place; then, with `side`, the per-layer token input of the step's
-    `tokens` on the residual just brought up to date: g = gelu_tanh(gate x) * table[token, offset ..],
-    y = proj g, residual += mult * y / sqrt(mean(y^2) + eps) * norm."""
+                    copy_dtype: torch.dtype | None = None) -> torch.Tensor | None:
+    """residual += mult * (first + second), in place.  copy_dtype: the residual as it is afterwards comes back once
+    more in that type (what a product that reads the residual takes as its input)."""
     _device_tensor(residual, "residual", torch.float32)
     _check_product(first, "first")
     rows, width = residual.shape
-    products = [first] + ([second] if second is not None else [])
-    for product in products:
+    for product in [first] + ([second] if second is not None else []):
         _check_product(product, "second")
         if (product.rows, product.cols) != (rows, width) or product.data.dtype != first.data.dtype:
             raise invalid_shape("residual_update: the sublayers' results do not fit the residual (or differ in type)")
+    copy = torch.empty((rows, width), dtype=copy_dtype, device=residual.device) if copy_dtype is not None else None
     if rows == 0:
-        return
-    args = [None, None, 0, 0, 0, None, None, None, F32, ctypes.c_float(1.0)]
-    if side is not None:
-        _device_tensor(tokens, "tokens", torch.int32)
-        for name in ("table", "gate", "proj", "norm"):
-            _device_tensor(getattr(side, name), name, side.table.dtype)
-        if (tokens.shape != (rows,) or side.table.dim() != 2 or side.offset < 0 or side.offset + side.dim > side.table.shape[1]
-                or side.gate.shape != (side.dim, width) or side.proj.shape != (width, side.dim) or side.norm.shape != (width,)):
-            raise invalid_shape("residual_update: the side input's tensors do not fit")
-        if width > RESIDUAL_UPDATE_MAX_WIDTH:
-            raise invalid_argument(f"residual_update: a side input goes with widths up to {RESIDUAL_UPDATE_MAX_WIDTH}")
-        if not side.eps > 0.0:
-            raise EngineError(ErrorCode.NUMERICAL, "a norm requires a positive epsilon")
-        args = [_ptr(tokens), _ptr(side.table), side.table.shape[1], side.offset, side.dim, _ptr(side.gate), _ptr(side.proj),
-                _ptr(side.norm), dtype_code(side.table.dtype), ctypes.c_float(side.eps)]
+        return copy
     _check(library().tlie_residual_update(_ptr(residual), _ptr(first.data), first.nsplit, ctypes.c_longlong(first.split_stride),
                                           _ptr(second.data if second is not None else None),
                                           second.nsplit if second is not None else 1,
                                           ctypes.c_longlong(second.split_stride if second is not None else 0),
-                                          dtype_code(first.data.dtype), ctypes.c_float(mult), rows, width, *args, _stream()),
+                                          dtype_code(first.data.dtype), ctypes.c_float(mult), ctypes.c_longlong(rows * width),
+                                          _ptr(copy), dtype_code(copy_dtype) if copy_dtype is not None else F32, _stream()),
            "residual_update")
+    return copy
+
+
+def side_gate(pre: Product, tokens: torch.Tensor, table: torch.Tensor, offset: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """g[t, j] = gelu_tanh(pre[t, j]) * table[tokens[t], offset + j], for the pre.cols columns of the table from `offset` on."""
+    _check_product(pre, "pre")
+    _device_tensor(tokens, "tokens", torch.int32)
+    _device_tensor(table, "table", (torch.float32, torch.bfloat16))
+    rows, dim = pre.rows, pre.cols
+    if tokens.shape != (rows,) or table.dim() != 2 or offset < 0 or offset + dim > table.shape[1]:
+        raise invalid_shape("side_gate: the table's columns or the tokens do not fit")
+    out = torch.empty((rows, dim), dtype=out_dtype, device=table.device)
+    if rows == 0:
+        return out
+    _check(library().tlie_side_gate(_ptr(pre.data), dtype_code(pre.data.dtype), pre.nsplit, ctypes.c_longlong(pre.split_stride),
+                                    _ptr(tokens), _ptr(table), dtype_code(table.dtype), table.shape[1], int(offset), dim, _ptr(out),
+                                    dtype_code(out_dtype), rows, _stream()), "side_gate")
+    return out
 
 
 def residual_inject(residual: torch.Tensor, tokens: torch.Tensor | None, table: torch.Tensor | None,

@@ -214,8 +214,9 @@ class SandwichNormBlock:
 class ParallelBlock:
     """x += scale * (mixer(norm(x)) + feed_forward(norm(x))): one norm, whose output both sublayers read; the
     feed-forward is optional.  After that, if the layer has one, an input that depends on the step's tokens (a part
-    of the "layer_input" table) joins the residual.  The block brings the residual up to date itself, in one kernel
-    for the two results, their factor and the layer input, and hands on nothing."""
+    of the "layer_input" table) joins the residual.  The block brings the residual up to date with the two results
+    itself, in one kernel; a layer input is normed before it joins and is handed on as a `NormedDelta`, which whoever
+    norms the residual next norms, adds and norms in one kernel."""
 
     def __init__(self, layer: LayerSpec, dtype, device):
         self.layer = layer
@@ -278,7 +279,14 @@ class ParallelBlock:
                 keep("mlp_output", fed.dense(torch.float32))
             if fed.data.dtype != mixed.data.dtype:       # (products of two kernels: as floats, so that one kernel adds both)
                 mixed, fed = ops.Product(mixed.dense(torch.float32).contiguous()), ops.Product(fed.dense(torch.float32).contiguous())
-        side = self.layer_input.side if self.layer_input is not None else None
-        ops.residual_update(residual, mixed, fed, self.scale, side=side, tokens=ctx.tokens if side is not None else None)
+        if self.layer_input is None:
+            ops.residual_update(residual, mixed, fed, self.scale)
+            keep("output", residual)
+            return None
+        copy = ops.residual_update(residual, mixed, fed, self.scale, copy_dtype=self.layer_input.copy_dtype())
+        waiting = self.layer_input.forward(residual, copy, ctx)
+        if trace is None:
+            return waiting
+        ops.norm_add_rmsnorm(residual, waiting.product, waiting.weight, waiting.eps, None, waiting.eps, self.dtype)
         keep("output", residual)
         return None

@@ -86,7 +86,7 @@ class MLSTM(Mixer):
         gates = ops.few_outputs(x, self.gates, self.gate_bias)
         keys, values = self.heads * self.d, self.heads * self.dv
         memory = ops.mlstm_scan(fused, 0, keys, 2 * keys, gates, binding.state, ctx.seq_start, ctx.seq_slot, self.heads, self.d,
-                                self.dv, self.cap, float(self.d) ** -0.5)
+                                self.dv, self.cap, float(self.d) ** -0.5, max_new=ctx.max_new)
         normed = ops.head_combine(memory, self.heads, self.dv, self.eps, self.dtype, weight=self.norm, gate=fused,
                                   gate_col=2 * keys + values)
         return self.o(normed)
