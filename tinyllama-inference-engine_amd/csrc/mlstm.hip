@@ -19,7 +19,7 @@
 // [tiles][dim * 64 (S, [d][lane]) + dim (n) + 1 (m, the first tile's only)].  Queries and keys of four tokens at a time
 // go through LDS (every lane needs all of them).
 //
-// A sequence that brings many tokens is taken in slices of 64 tokens that run side by side: every slice is walked
+// A sequence that brings many tokens is taken in slices of 32 tokens that run side by side: every slice is walked
 // from a memory of zero and leaves where it ends and the product of its keeps (S' = keep S + take k v^T is linear
 // in S); a second kernel gives every slice its start, start(c + 1) = keeps(c) * start(c) + end(c), and the state its
 // new value; a third walks every slice again from its start and writes the results.
@@ -27,7 +27,7 @@
 
 namespace tlie {
 
-constexpr int kMlstmBatch = 4, kMlstmSlice = 64;
+constexpr int kMlstmBatch = 4, kMlstmSlice = 32;
 
 // gates: float [tokens, 2 * heads] (input gates' pre-activations, then forget gates'); values: float [tokens, heads, 4]
 // (keep, take, exp(-m), unused).  One wave per (sequence, head); m is the state's, read and written here only.
@@ -35,7 +35,6 @@ __global__ void __launch_bounds__(64)
 mlstm_gates_kernel(const float* __restrict__ gates, float* __restrict__ values, float* __restrict__ state,
                    const int* __restrict__ seq_start, const int* __restrict__ seq_slot, int heads, size_t head_floats,
                    size_t m_offset, float cap) {
-  __shared__ float log_i[64], log_f[64], maxima[65];
   const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int slot = seq_slot[seq];
   if (slot < 0) return;
@@ -51,21 +50,26 @@ mlstm_gates_kernel(const float* __restrict__ gates, float* __restrict__ values, 
       const float x = cap * tanhf(gates[static_cast<size_t>(t) * 2 * heads + heads + h] / cap);
       fg = fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
     }
-    __syncthreads();
-    log_i[lane] = ig, log_f[lane] = fg;
-    __syncthreads();
-    if (lane == 0) {                                   // the running maximum, token by token
-      maxima[0] = m;
-      for (int j = 0; j < count; ++j) maxima[j + 1] = fmaxf(log_f[j] + maxima[j], log_i[j]);
+    // m' = max(m + f, i) token by token is a chain of the maps m -> max(m + F, I); two in a row are one of the same
+    // kind, (F1 + F2, max(I1 + F2, I2)), so the wave forms every token's map of all tokens up to it in six steps
+    float F = lane < count ? fg : 0.f, I = lane < count ? ig : -INFINITY;
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+      const float Fb = __shfl_up(F, offset, 64), Ib = __shfl_up(I, offset, 64);
+      if (lane >= offset) {
+        I = fmaxf(Ib + F, I);
+        F = Fb + F;
+      }
     }
-    __syncthreads();
+    const float after = fmaxf(m + F, I);               // m after this lane's token
+    float before = __shfl_up(after, 1, 64);
+    if (lane == 0) before = m;
     if (lane < count) {
-      const float before = maxima[lane], after = maxima[lane + 1];
       float4 out;
       out.x = expf(fg + before - after), out.y = expf(ig - after), out.z = expf(-after), out.w = 0.f;
       *reinterpret_cast<float4*>(values + (static_cast<size_t>(t) * heads + h) * 4) = out;
     }
-    m = maxima[count];
+    m = __shfl(after, count - 1, 64);
   }
   if (lane == 0) *m_place = m;
 }
@@ -109,28 +113,46 @@ mlstm_scan_kernel(const D* __restrict__ fused, int nsplit, size_t split_stride, 
   }
   float keeps = 1.f;
 
-  for (int t0 = first; t0 < last; t0 += kMlstmBatch) {
+  // a batch of tokens is asked for while the batch before it is worked on: its queries, keys, values and gates wait
+  // in registers (a wave is alone on its SIMD where slices are few, and nothing else would hide the loads' way)
+  float rq[kMlstmBatch][NJ], rk[kMlstmBatch][NJ], rv[kMlstmBatch];
+  float4 rg[kMlstmBatch];
+  auto fetch = [&](int t0) {
     const int nb = min(kMlstmBatch, last - t0);
-    __syncthreads();                                   // the batch before has been read
-    float vv[kMlstmBatch], keep[kMlstmBatch], take[kMlstmBatch], floor_[kMlstmBatch];
 #pragma unroll
     for (int b = 0; b < kMlstmBatch; ++b) {
       const D* row = fused + static_cast<size_t>(t0 + b) * row_width;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const int d = lane + 64 * j;
+        const bool there = b < nb && d < dim;
+        rq[b][j] = MODE != 1 && there ? sum_splits(row + q_col + h * dim + d, nsplit, split_stride) * q_scale : 0.f;
+        rk[b][j] = there ? sum_splits(row + k_col + h * dim + d, nsplit, split_stride) : 0.f;
+      }
+      rv[b] = b < nb && live ? sum_splits(row + v_col + h * vdim + col, nsplit, split_stride) : 0.f;
+      rg[b] = b < nb ? *reinterpret_cast<const float4*>(values + (static_cast<size_t>(t0 + b) * heads + h) * 4)
+                     : make_float4(1.f, 0.f, 1.f, 0.f);
+    }
+  };
+  fetch(first);
+  for (int t0 = first; t0 < last; t0 += kMlstmBatch) {
+    const int nb = min(kMlstmBatch, last - t0);
+    __syncthreads();                                   // the batch before has been read
+    float vv[kMlstmBatch], keep[kMlstmBatch], take[kMlstmBatch], floor_[kMlstmBatch];
+#pragma unroll
+    for (int b = 0; b < kMlstmBatch; ++b) {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int d = lane + 64 * j;
         if (d < DMAX) {
-          const bool there = b < nb && d < dim;
-          if (MODE != 1) qs[b][d] = there ? sum_splits(row + q_col + h * dim + d, nsplit, split_stride) * q_scale : 0.f;
-          ks[b][d] = there ? sum_splits(row + k_col + h * dim + d, nsplit, split_stride) : 0.f;
+          if (MODE != 1) qs[b][d] = rq[b][j];
+          ks[b][d] = rk[b][j];
         }
       }
-      vv[b] = b < nb && live ? sum_splits(row + v_col + h * vdim + col, nsplit, split_stride) : 0.f;
-      const float4 gate = b < nb ? *reinterpret_cast<const float4*>(values + (static_cast<size_t>(t0 + b) * heads + h) * 4)
-                                 : make_float4(1.f, 0.f, 1.f, 0.f);
-      keep[b] = gate.x, take[b] = gate.y, floor_[b] = gate.z;
+      vv[b] = rv[b], keep[b] = rg[b].x, take[b] = rg[b].y, floor_[b] = rg[b].z;
     }
     __syncthreads();
+    if (t0 + kMlstmBatch < last) fetch(t0 + kMlstmBatch);
 #pragma unroll
     for (int b = 0; b < kMlstmBatch; ++b) {
       if (b >= nb) break;                              // (the same for the whole wave)
@@ -217,7 +239,7 @@ using namespace tlie;
 // forget gates' pre-activations; values: float [tokens, heads, 4], scratch for what the gates become; state: float
 // [slots, heads, tiles, dim * 64 + dim + 1], tiles = ceil(vdim / 64); seq_start [sequences + 1], seq_slot [sequences]
 // (negative: skipped); out: float [tokens, heads * vdim].  slices 0: every sequence's tokens are walked in order;
-// slices > 0 (at least ceil(most tokens of a sequence / 64)): in slices of 64 tokens side by side, with parts: float
+// slices > 0 (at least ceil(most tokens of a sequence / 32)): in slices of 32 tokens side by side, with parts: float
 // [sequences, slices, heads, tiles, dim * 64 + dim + 1] as scratch.
 extern "C" int tlie_mlstm_scan(const void* fused, int dtype, int nsplit, long long split_stride, int row_width, int q_col,
                                int k_col, int v_col, const float* gates, float* values, float* state, const int* seq_start,

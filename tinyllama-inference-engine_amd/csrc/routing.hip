@@ -20,15 +20,35 @@ few_outputs_kernel(const X* __restrict__ x, const W* __restrict__ w, const W* __
   extern __shared__ float sums[];                      // outputs
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const X* row = x + static_cast<size_t>(t) * inner;
+  // (eight inner indices a lane and load where the rows allow it: a wave then asks for a kilobyte or two at once, and a
+  // sum of 2048 terms waits for memory four times, not sixteen)
+  const bool wide = (inner & 7) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 31) == 0;
   for (int n = wave; n < outputs; n += 4) {
     const W* weights = w + static_cast<size_t>(n) * inner;
     float a = 0.f, b = 0.f;
-    int k = lane;
-    for (; k + 64 < inner; k += 128) {
-      a += to_float(row[k]) * to_float(weights[k]);
-      b += to_float(row[k + 64]) * to_float(weights[k + 64]);
+    if (wide) {
+#pragma unroll 2
+      for (int k = lane * 8; k < inner; k += 512) {
+        float xv[8], wv[8];
+        load8(row + k, xv);
+        load8(weights + k, wv);
+        a += xv[0] * wv[0];
+        b += xv[1] * wv[1];
+        a += xv[2] * wv[2];
+        b += xv[3] * wv[3];
+        a += xv[4] * wv[4];
+        b += xv[5] * wv[5];
+        a += xv[6] * wv[6];
+        b += xv[7] * wv[7];
+      }
+    } else {
+      int k = lane;
+      for (; k + 64 < inner; k += 128) {
+        a += to_float(row[k]) * to_float(weights[k]);
+        b += to_float(row[k + 64]) * to_float(weights[k + 64]);
+      }
+      if (k < inner) a += to_float(row[k]) * to_float(weights[k]);
     }
-    if (k < inner) a += to_float(row[k]) * to_float(weights[k]);
     float total = wave_sum(a + b);
     if (bias != nullptr) total += to_float(bias[n]);
     if (top <= 0) {

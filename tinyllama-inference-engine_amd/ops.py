@@ -616,8 +616,8 @@ def head_combine(a: torch.Tensor, heads: int, value_dim: int, eps: float, out_dt
 
 
 MLSTM_MAX_DIM = 256            # the largest query/key size of a head that the matrix-memory kernel keeps in registers
-MLSTM_SLICE = 64               # tokens of a slice of the sliced walk (the kernel's kMlstmSlice)
-MLSTM_SLICED_FROM = 192        # tokens a sequence brings from which the sliced walk pays (two walks of a slice and a carry)
+MLSTM_SLICE = 32               # tokens of a slice of the sliced walk (the kernel's kMlstmSlice)
+MLSTM_SLICED_FROM = 96         # tokens a sequence brings from which the sliced walk pays (two walks of a slice and a carry)
 
 
 def mlstm_state_shape(heads: int, dim: int, value_dim: int) -> tuple[int, ...]:
