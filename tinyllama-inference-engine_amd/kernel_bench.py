@@ -344,5 +344,143 @@ def bench_design_kernels(sizes: dict, batch: int = 8, context: int = 2048, promp
 
 def bench_raketar_kernels(sizes: dict, batch: int = 8, context: int = 2048, prompt: int = 2048, samples: int = 10, device="cuda:0",
                           hbm_gbs: float = 8000.0, mfma_tflops: float = 2500.0) -> list[dict]:
-    """The kernels that the Raketar decoder adds, each alone at a layer's sizes (filled in below)."""
-    return []
+    """The kernels that the Raketar decoder adds, each alone at a layer's sizes, for a decode step of `batch` requests at
+    `context` positions and a prompt step of `prompt` tokens, each beside the like kernel of the Llama decoder at the
+    same sizes; every row carries the fraction of the roofline its bytes or flops reach (`frac`: of `hbm_gbs` for rows
+    with bytes, of `mfma_tflops` for rows with flops).
+    sizes: width, ff, heads, kv_heads, dim, vdim (differential attention), llama_heads, llama_kv_heads; memory_heads,
+    memory_dim, memory_vdim; experts, top, expert_ff, shared_ff; side."""
+    device = torch.device(device)
+    torch.cuda.set_device(device)
+    bf, f32 = torch.bfloat16, torch.float32
+    width, ff = sizes["width"], sizes["ff"]
+    H, G, d, dv = sizes["heads"], sizes["kv_heads"], sizes["dim"], sizes["vdim"]
+    lq, lkv = sizes["llama_heads"], sizes["llama_kv_heads"]
+    mh, md, mv = sizes["memory_heads"], sizes["memory_dim"], sizes["memory_vdim"]
+    experts, top, eff, sff, side = sizes["experts"], sizes["top"], sizes["expert_ff"], sizes["shared_ff"], sizes["side"]
+    page_size, rows = 16, []
+    units = int(torch.cuda.get_device_properties(device).multi_processor_count)
+
+    def rand(*shape, scale=0.02, dtype=bf):
+        return (torch.randn(shape, device=device, dtype=f32) * scale).to(dtype)
+
+    def row(name, times, read_bytes=0, flops=0):
+        entry = _row(name, times, read_bytes, flops)
+        if read_bytes:
+            entry["frac"] = round(entry["gbs"] / hbm_gbs, 3)
+        elif flops:
+            entry["frac"] = round(entry["tflops"] / mfma_tflops, 4)
+        rows.append(entry)
+
+    def ints(values):
+        return torch.tensor(values, dtype=torch.int32, device=device)
+
+    for label, tokens, seqs in ((f"decode b{batch}", batch, batch), (f"prompt {prompt}", prompt, 1)):
+        if tokens <= 0:
+            continue
+        decode = seqs == tokens
+        length = context if decode else prompt
+        blocks = (length + page_size - 1) // page_size
+        table = torch.arange(seqs * blocks, dtype=torch.int32, device=device).view(seqs, blocks).contiguous()
+        if decode:
+            positions = torch.full((tokens,), length - 1, dtype=torch.int32, device=device)
+            token_seq, seq_start = ints(list(range(tokens))), ints(list(range(tokens + 1)))
+            host = {"seq_start": np.arange(tokens + 1, dtype=np.int32), "seq_len": np.full(tokens, length, dtype=np.int32)}
+        else:
+            positions = torch.arange(tokens, dtype=torch.int32, device=device)
+            token_seq, seq_start = torch.zeros(tokens, dtype=torch.int32, device=device), ints([0, tokens])
+            host = {"seq_start": np.asarray([0, tokens], dtype=np.int32), "seq_len": np.asarray([tokens], dtype=np.int32)}
+        slot_map = (table[token_seq.long(), (positions // page_size).long()] * page_size + positions % page_size).to(torch.int32).contiguous()
+        seq_slot = ints(list(range(seqs)))
+        ids = torch.randint(0, 1000, (tokens,), device=device, dtype=torch.int32)
+        ctx = SimpleNamespace(max_new=1 if decode else tokens, num_seqs=seqs, num_tokens=tokens, max_context=length, scratch={},
+                              tile_owner=None, compute_units=units, host=host, tokens=positions)
+        keys_seen = length if decode else (length + 1) / 2            # keys a token sees on average
+        # ---- attention: two maps a head over shared values, beside the plain causal one of as many query heads -------
+        parts = dv // d
+        cache = rand(seqs * blocks, 2, lkv, page_size * d, scale=0.5)
+        q = rand(tokens, lq * d, scale=1.0)
+        tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, lq // lkv, lkv, d)
+        times = _timed(lambda i: ops.attention_mfma(q, cache, table, tiles, positions, lq, lkv, d, None, d ** -0.5, nsplit, split_len,
+                                                    col_tiles, waves, shared), 8, samples)
+        cache_bytes, flops = seqs * length * lkv * 2 * d * 2, 4.0 * tokens * lq * d * keys_seen
+        row(f"{label}: attention, causal (Llama's), {lq} heads of {d} on {lkv}", times, cache_bytes if decode else 0, 0 if decode else flops)
+        ctx.scratch = {}
+        cache2 = rand(seqs * blocks, G, page_size * (2 * d + dv), scale=0.5)
+        q2 = rand(tokens, 2 * H * d, scale=1.0)
+        tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, H // G, 2 * G * parts, d)
+        times = _timed(lambda i: ops.attention_mfma(q2, cache2, table, tiles, positions, 2 * H * parts, 2 * G * parts, d, None, d ** -0.5,
+                                                    nsplit, split_len, col_tiles, waves, shared, planes=(parts, 2 * parts, parts),
+                                                    float_out=True), 8, samples)
+        cache_bytes = seqs * length * G * (2 * d + dv) * 2
+        flops = 2.0 * tokens * 2 * H * (d + dv) * keys_seen             # scores once a map, values of dv
+        row(f"{label}: attention, two maps of {H} heads of {d} on {G} groups, values of {dv}", times, cache_bytes if decode else 0,
+            0 if decode else flops)
+        attended = rand(tokens, 2 * H * dv, scale=1.0, dtype=f32)
+        fused = ops.Product(rand(tokens, 2 * H * d + 2 * G * d + G * dv + H * dv, scale=1.0), 1)
+        times = _timed(lambda i: ops.head_combine(attended, H, dv, 1e-5, bf, pair_group=H // G, pair_lambda=0.3, mult=0.5, gate=fused,
+                                                  gate_col=fused.cols - H * dv, parts=parts), 8, samples)
+        row(f"{label}: difference of the maps, norm and gate", times, tokens * H * dv * (8 + 2 + 2))
+        times = _timed(lambda i: ops.qkv_place(fused, positions, slot_map, torch.ones(d // 2, device=device), d, cache2, 2 * H, 2 * G, d, dv,
+                                               bf, value_heads=G, extra_cols=H * dv), 8, samples)
+        row(f"{label}: placement of q, k, v (shared value heads)", times, tokens * (2 * H * d * 2 + 2 * G * d + G * dv) * 2 * 2)
+        qkv = ops.Product(rand(tokens, (lq + 2 * lkv) * d, scale=1.0), 1)
+        times = _timed(lambda i: ops.rope_cache(qkv, positions, slot_map, torch.ones(d // 2, device=device), d, cache, lq, lkv, d, bf), 8, samples)
+        row(f"{label}: rotation + cache write (Llama's)", times, tokens * (lq * 2 + 2 * lkv) * d * 2 * 2)
+        # ---- the matrix memory -------------------------------------------------------------------------------------
+        memory_in = ops.Product(rand(tokens, 2 * mh * md + 2 * mh * mv, scale=1.0), 1)
+        gates = rand(tokens, 2 * mh, scale=1.0, dtype=f32) + 3.0
+        state = torch.zeros((seqs, *ops.mlstm_state_shape(mh, md, mv)), dtype=f32, device=device)
+        times = _timed(lambda i: ops.mlstm_scan(memory_in, 0, mh * md, 2 * mh * md, gates, state, seq_start, seq_slot, mh, md, mv, 15.0,
+                                                md ** -0.5, max_new=ctx.max_new), 8, samples)
+        state_bytes = seqs * mh * md * mv * 4 * 2
+        # a token: S = keep S + k v^T and S^T q, 4 flops an element of S (the sliced walk does the first half twice)
+        row(f"{label}: matrix memory, {mh} heads of {md} x {mv} (gates, walk)", times, state_bytes if decode else 0,
+            0 if decode else 4.0 * tokens * mh * md * mv)
+        memory_out = rand(tokens, mh * mv, scale=1.0, dtype=f32)
+        weight = rand(mh * mv, scale=1.0)
+        times = _timed(lambda i: ops.head_combine(memory_out, mh, mv, 1e-5, bf, weight=weight, gate=memory_in, gate_col=2 * mh * md + mh * mv),
+                       8, samples)
+        row(f"{label}: the memory heads' norm and gate", times, tokens * mh * mv * (4 + 2 + 2))
+        x = rand(tokens, width, scale=1.0)
+        gate_w, gate_b = rand(2 * mh, width), rand(2 * mh)
+        times = _timed(lambda i: ops.few_outputs(x, gate_w, gate_b), 8, samples)
+        row(f"{label}: the gates' product, float sums ({2 * mh} outputs)", times, (tokens + 2 * mh) * width * 2)
+        # ---- the routed feed-forward -------------------------------------------------------------------------------
+        router = rand(experts, width)
+        times = _timed(lambda i: ops.few_outputs(x, router, top=top), 8, samples)
+        row(f"{label}: router, {top} of {experts}", times, (tokens + experts) * width * 2)
+        inter = experts * eff + sff
+        scale = ops.few_outputs(x, router, top=top)
+        gate_up = ops.Product(rand(tokens, 2 * inter, scale=1.0), 1)
+        times = _timed(lambda i: ops.routed_gate(gate_up, scale, eff, bf), 4, samples)
+        row(f"{label}: gate of the routed feed-forward (all experts' columns)", times, tokens * inter * 6)
+        dense_up = ops.Product(rand(tokens, 2 * ff, scale=1.0), 1)
+        times = _timed(lambda i: ops.silu_mul(dense_up, bf, interleaved=True), 4, samples)
+        row(f"{label}: SiLU gate (Llama's)", times, tokens * ff * 6)
+        if not decode:
+            from .parts.linear import Linear
+            for name, out_features, in_features, useful in (
+                    ("routed gate/up, all experts", 2 * inter, width, 2 * (top * eff + sff)), ("routed down, all experts", width, inter, None),
+                    ("dense gate/up (Llama's)", 2 * ff, width, 2 * ff), ("dense down (Llama's)", width, ff, None)):
+                linear = Linear(rand(out_features, in_features), None, bf)
+                operand = rand(tokens, in_features, scale=1.0)
+                times = _timed(lambda i: linear(operand), 4, samples)
+                used = useful if useful is not None else out_features
+                inner = in_features if useful is not None else (top * eff + sff if "routed" in name else ff)
+                row(f"{label}: {name} (flops of the experts in use)", times, 0, 2.0 * tokens * used * inner)
+        # ---- the residual and the token input ----------------------------------------------------------------------
+        residual = rand(tokens, width, scale=1.0, dtype=f32)
+        first, second = ops.Product(rand(tokens, width, scale=1.0), 1), ops.Product(rand(tokens, width, scale=1.0), 1)
+        times = _timed(lambda i: ops.residual_update(residual, first, second, 0.5, copy_dtype=bf), 8, samples)
+        row(f"{label}: residual += both sublayers, copy for the token input", times, tokens * width * (4 + 4 + 2 + 2 + 2))
+        norm_w = rand(width, scale=1.0)
+        times = _timed(lambda i: ops.norm_add_rmsnorm(residual, first, norm_w, 1e-5, norm_w, 1e-5, bf), 8, samples)
+        row(f"{label}: token input normed, added, next norm", times, tokens * width * (4 + 4 + 2 + 2))
+        times = _timed(lambda i: ops.add_rmsnorm(residual, first, norm_w, 1e-5, bf), 8, samples)
+        row(f"{label}: add + norm (Llama's)", times, tokens * width * (4 + 4 + 2 + 2))
+        pre = ops.Product(rand(tokens, side, scale=1.0), 1)
+        side_table = rand(1000, 4 * side, scale=1.0)
+        times = _timed(lambda i: ops.side_gate(pre, ids, side_table, side, bf), 8, samples)
+        row(f"{label}: token input's gate", times, tokens * side * 6)
+    return rows
