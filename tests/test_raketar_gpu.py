@@ -553,3 +553,41 @@ def test_long_decoding_keeps_to_the_plain_implementation(setups):
         engine = new_engine(setup, dtype)
         got = run_cut(engine, "a", tokens, [6] + [1] * 400)
         assert_rows(got, want, TOLERANCE[dtype], f"{dtype}")
+
+
+def test_the_command_line_and_the_replay_program_run_the_design(setups, tmp_path):
+    """`generate` and `logits` of the framework's command line, and a trace of steps through `bin/trace_run` (a portion
+    beside a single token, a request that ends and whose slot and pages are used again), on a model of this design."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    setup = setups("T")
+    vocab = CONFIGS["T"]["vocab"]
+    tokens, other = tokens_of(61, 40, vocab), tokens_of(62, 21, vocab)
+    prompt = "ids:" + ",".join(str(token) for token in tokens[:9])
+    cli = [sys.executable, os.path.join(root, "bin", "tinyllama_amd")]
+    run = subprocess.run(cli + ["generate", setup["folder"], prompt, "6", "--dtype", "float32"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    assert json.loads(run.stdout)["generated_tokens"] == plain_generate_greedy(setup["raw"], setup["weights"], tokens[:9], 6)
+    run = subprocess.run(cli + ["logits", setup["folder"], prompt, "--dtype", "float32"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    assert_rows(torch.tensor(json.loads(run.stdout)["logits"])[None], plain_logits(setup, tokens[:9])[-1:], TOLERANCE["float32"], "logits")
+    lines = [{"step": 0, "entries": [{"id": "a", "tokens": tokens[:30], "want": [0, 29]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": tokens[30:31], "want": [0]}, {"id": "b", "tokens": other, "want": [20]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "c", "tokens": other[:7], "want": []}], "end": []},
+             {"step": 3, "entries": [{"id": "a", "tokens": tokens[31:], "want": [8]}, {"id": "c", "tokens": other[7:], "want": [13]}], "end": ["a", "c"]}]
+    for dtype in DTYPES:
+        out = tmp_path / dtype
+        run = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", setup["folder"], "--dtype", dtype,
+                              "--out", str(out), "--max-tokens", "128", "--max-requests", "2"],
+                             input="".join(json.dumps(line) + "\n" for line in lines), capture_output=True, text=True, timeout=300)
+        assert run.returncode == 0 and run.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "3"], run.stderr
+        assert not (out / "2.f32").exists()
+        read = lambda step: torch.from_numpy(numpy.fromfile(out / f"{step}.f32", dtype="<f4").reshape(-1, vocab))
+        want, want_other = plain_logits(setup, tokens), plain_logits(setup, other)
+        assert_rows(read(0), want[[0, 29]], TOLERANCE[dtype], f"{dtype} step 0")
+        assert_rows(read(1), torch.stack([want[30], want_other[20]]), TOLERANCE[dtype], f"{dtype} step 1")
+        assert_rows(read(3), torch.stack([want[39], want_other[20]]), TOLERANCE[dtype], f"{dtype} step 3")
