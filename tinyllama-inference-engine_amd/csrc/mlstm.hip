@@ -78,17 +78,21 @@ mlstm_gates_kernel(const float* __restrict__ gates, float* __restrict__ values, 
 // MODE 1: a slice from zero; no results; where it ends and the product of its keeps go to `parts`.
 // MODE 2: a slice from the start that `parts` now holds for it; results written.
 // parts: float [sequences, slices, heads, tiles, dim * 64 + dim + 1] (S, n, the product of the slice's keeps).
-template <typename D, int DMAX, int MODE>
-__global__ void __launch_bounds__(64)
+// A workgroup has WAVES waves; wave w keeps dims w * DW .. (w + 1) * DW of its lanes' columns of S (and of n), so that
+// a column of up to 256 dims stays in registers; the waves' parts of a token's sums meet in LDS, once a batch.
+template <typename D, int DW, int WAVES, int MODE>
+__global__ void __launch_bounds__(64 * WAVES)
 mlstm_scan_kernel(const D* __restrict__ fused, int nsplit, size_t split_stride, int row_width, int q_col, int k_col,
                   int v_col, const float* __restrict__ values, float* __restrict__ state, float* __restrict__ parts,
                   const int* __restrict__ seq_start, const int* __restrict__ seq_slot, float* __restrict__ out, int heads,
                   int dim, int vdim, int tiles, int slices, float q_scale) {
-  constexpr int NJ = DMAX >= 64 ? DMAX / 64 : 1;
+  constexpr int NJ = DW >= 64 ? DW / 64 : 1, DMAX = DW * WAVES;
   __shared__ __attribute__((aligned(16))) float qs[kMlstmBatch][DMAX];
   __shared__ __attribute__((aligned(16))) float ks[kMlstmBatch][DMAX];
+  __shared__ float met[WAVES][kMlstmBatch][65];        // a wave's part of a token's S^T q (64 lanes) and of n . q
   const int seq = MODE == 0 ? blockIdx.x : blockIdx.x / slices, slice = MODE == 0 ? 0 : blockIdx.x % slices;
-  const int h = blockIdx.y, tile = blockIdx.z, lane = threadIdx.x;
+  const int h = blockIdx.y, tile = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int base = wave * DW;                          // this wave's first dim
   const int slot = seq_slot[seq];
   if (slot < 0) return;                                // a sequence that pads a recorded step: no state is its own
   int first = seq_start[seq], last = seq_start[seq + 1];
@@ -102,14 +106,14 @@ mlstm_scan_kernel(const D* __restrict__ fused, int nsplit, size_t split_stride, 
   const size_t tile_floats = static_cast<size_t>(dim) * 64 + dim + 1;
   float* st = MODE == 0 ? state + ((static_cast<size_t>(slot) * heads + h) * tiles + tile) * tile_floats
                         : parts + (((static_cast<size_t>(seq) * slices + slice) * heads + h) * tiles + tile) * tile_floats;
-  float S[DMAX];
+  float S[DW];
   float n[NJ];
 #pragma unroll
-  for (int d = 0; d < DMAX; ++d) S[d] = MODE != 1 && d < dim ? st[d * 64 + lane] : 0.f;
+  for (int d = 0; d < DW; ++d) S[d] = MODE != 1 && base + d < dim ? st[(base + d) * 64 + lane] : 0.f;
 #pragma unroll
   for (int j = 0; j < NJ; ++j) {
-    const int d = lane + 64 * j;
-    n[j] = MODE != 1 && d < dim ? st[static_cast<size_t>(dim) * 64 + d] : 0.f;
+    const int d = base + lane + 64 * j;
+    n[j] = MODE != 1 && lane + 64 * j < DW && d < dim ? st[static_cast<size_t>(dim) * 64 + d] : 0.f;
   }
   float keeps = 1.f;
 
@@ -124,8 +128,8 @@ mlstm_scan_kernel(const D* __restrict__ fused, int nsplit, size_t split_stride, 
       const D* row = fused + static_cast<size_t>(t0 + b) * row_width;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        const int d = lane + 64 * j;
-        const bool there = b < nb && d < dim;
+        const int d = base + lane + 64 * j;
+        const bool there = b < nb && lane + 64 * j < DW && d < dim;
         rq[b][j] = MODE != 1 && there ? sum_splits(row + q_col + h * dim + d, nsplit, split_stride) * q_scale : 0.f;
         rk[b][j] = there ? sum_splits(row + k_col + h * dim + d, nsplit, split_stride) : 0.f;
       }
@@ -143,31 +147,32 @@ mlstm_scan_kernel(const D* __restrict__ fused, int nsplit, size_t split_stride, 
     for (int b = 0; b < kMlstmBatch; ++b) {
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        const int d = lane + 64 * j;
-        if (d < DMAX) {
-          if (MODE != 1) qs[b][d] = rq[b][j];
-          ks[b][d] = rk[b][j];
+        if (lane + 64 * j < DW) {
+          if (MODE != 1) qs[b][base + lane + 64 * j] = rq[b][j];
+          ks[b][base + lane + 64 * j] = rk[b][j];
         }
       }
       vv[b] = rv[b], keep[b] = rg[b].x, take[b] = rg[b].y, floor_[b] = rg[b].z;
     }
     __syncthreads();
     if (t0 + kMlstmBatch < last) fetch(t0 + kMlstmBatch);
+    float top[kMlstmBatch], under[kMlstmBatch];         // this wave's part of S^T q and of n . q, a token each
 #pragma unroll
     for (int b = 0; b < kMlstmBatch; ++b) {
-      if (b >= nb) break;                              // (the same for the whole wave)
+      top[b] = under[b] = 0.f;
+      if (b >= nb) continue;                           // (the same for the whole wave)
       const float tv = take[b] * vv[b];
       float acc = 0.f;
 #pragma unroll
-      for (int d0 = 0; d0 < DMAX; d0 += 4) {
-        if (d0 < dim) {                                // (entries from dim on are zeros in LDS and stay zeros in S)
-          const float4 k4 = *reinterpret_cast<const float4*>(&ks[b][d0]);
+      for (int d0 = 0; d0 < DW; d0 += 4) {
+        if (base + d0 < dim) {                         // (entries from dim on are zeros in LDS and stay zeros in S)
+          const float4 k4 = *reinterpret_cast<const float4*>(&ks[b][base + d0]);
           S[d0 + 0] = keep[b] * S[d0 + 0] + k4.x * tv;
           S[d0 + 1] = keep[b] * S[d0 + 1] + k4.y * tv;
           S[d0 + 2] = keep[b] * S[d0 + 2] + k4.z * tv;
           S[d0 + 3] = keep[b] * S[d0 + 3] + k4.w * tv;
           if (MODE != 1) {
-            const float4 q4 = *reinterpret_cast<const float4*>(&qs[b][d0]);
+            const float4 q4 = *reinterpret_cast<const float4*>(&qs[b][base + d0]);
             acc += S[d0 + 0] * q4.x;
             acc += S[d0 + 1] * q4.y;
             acc += S[d0 + 2] * q4.z;
@@ -178,31 +183,46 @@ mlstm_scan_kernel(const D* __restrict__ fused, int nsplit, size_t split_stride, 
       float partial = 0.f;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        const int d = lane + 64 * j;
-        if (d < DMAX) {
-          n[j] = keep[b] * n[j] + take[b] * ks[b][d];
-          if (MODE != 1) partial += n[j] * qs[b][d];
+        if (lane + 64 * j < DW) {
+          n[j] = keep[b] * n[j] + take[b] * ks[b][base + lane + 64 * j];
+          if (MODE != 1) partial += n[j] * qs[b][base + lane + 64 * j];
         }
       }
-      if (MODE == 1) {
-        keeps *= keep[b];
-      } else {
-        const float nq = wave_sum(partial);
-        const float bottom = fmaxf(fabsf(nq), floor_[b]) + 1e-6f;
-        if (live) out[(static_cast<size_t>(t0 + b) * heads + h) * vdim + col] = acc / bottom;
+      if (MODE == 1) keeps *= keep[b];
+      else top[b] = acc, under[b] = wave_sum(partial);
+    }
+    if (MODE == 1) continue;
+    if (WAVES > 1) {
+#pragma unroll
+      for (int b = 0; b < kMlstmBatch; ++b) {
+        met[wave][b][lane] = top[b];
+        if (lane == 0) met[wave][b][64] = under[b];
       }
+      __syncthreads();
+      if (wave != 0) continue;
+#pragma unroll
+      for (int b = 0; b < kMlstmBatch; ++b) {
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) top[b] += met[w][b][lane], under[b] += met[w][b][64];
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < kMlstmBatch; ++b) {
+      if (b >= nb) continue;
+      const float bottom = fmaxf(fabsf(under[b]), floor_[b]) + 1e-6f;
+      if (live) out[(static_cast<size_t>(t0 + b) * heads + h) * vdim + col] = top[b] / bottom;
     }
   }
   if (MODE == 2) return;
 #pragma unroll
-  for (int d = 0; d < DMAX; ++d)
-    if (d < dim) st[d * 64 + lane] = S[d];
+  for (int d = 0; d < DW; ++d)
+    if (base + d < dim) st[(base + d) * 64 + lane] = S[d];
 #pragma unroll
   for (int j = 0; j < NJ; ++j) {
-    const int d = lane + 64 * j;
-    if (d < dim) st[static_cast<size_t>(dim) * 64 + d] = n[j];
+    const int d = base + lane + 64 * j;
+    if (lane + 64 * j < DW && d < dim) st[static_cast<size_t>(dim) * 64 + d] = n[j];
   }
-  if (MODE == 1 && lane == 0) st[static_cast<size_t>(dim) * 64 + dim] = keeps;
+  if (MODE == 1 && threadIdx.x == 0) st[static_cast<size_t>(dim) * 64 + dim] = keeps;
 }
 
 // Every slice's start from the state and the slices before it, in place: where a slice's end stood its start stands
@@ -256,13 +276,13 @@ extern "C" int tlie_mlstm_scan(const void* fused, int dtype, int nsplit, long lo
   hipLaunchKernelGGL(mlstm_gates_kernel, dim3(sequences, heads), dim3(64), 0, s, gates, values, state, seq_start, seq_slot,
                      heads, tiles * tile_floats, tile_floats - 1, cap);
   if (launch_status() != kOk) return kLaunchFailed;
-#define TLIE_LAUNCH(D, DMAX, MODE, GRID)                                                                              \
-  hipLaunchKernelGGL((mlstm_scan_kernel<D, DMAX, MODE>), GRID, dim3(64), 0, s, (const D*)fused, nsplit,                \
+#define TLIE_LAUNCH(D, DW, WAVES, MODE, GRID)                                                                         \
+  hipLaunchKernelGGL((mlstm_scan_kernel<D, DW, WAVES, MODE>), GRID, dim3(64 * WAVES), 0, s, (const D*)fused, nsplit,   \
                      (size_t)split_stride, row_width, q_col, k_col, v_col, values, state, parts, seq_start, seq_slot,  \
                      out, heads, dim, vdim, tiles, slices, q_scale)
 #define TLIE_SIZES(D, MODE, GRID)                                                                                     \
-  if (dim <= 32) TLIE_LAUNCH(D, 32, MODE, GRID); else if (dim <= 64) TLIE_LAUNCH(D, 64, MODE, GRID);                  \
-  else if (dim <= 128) TLIE_LAUNCH(D, 128, MODE, GRID); else TLIE_LAUNCH(D, 256, MODE, GRID)
+  if (dim <= 32) TLIE_LAUNCH(D, 32, 1, MODE, GRID); else if (dim <= 64) TLIE_LAUNCH(D, 64, 1, MODE, GRID);            \
+  else if (dim <= 128) TLIE_LAUNCH(D, 64, 2, MODE, GRID); else TLIE_LAUNCH(D, 128, 2, MODE, GRID)
 #define TLIE_TYPES(MODE, GRID)                                                                                        \
   if (dtype == kF32) { TLIE_SIZES(float, MODE, GRID); }                                                               \
   else if (dtype == kBF16) { TLIE_SIZES(bf16, MODE, GRID); }                                                          \
