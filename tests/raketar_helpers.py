@@ -68,7 +68,8 @@ TOLERANCE = {"float32": 3e-5, "bfloat16": 1.5e-1}
 SINGLE_LAYER_TOLERANCE = {"float32": 3e-5, "bfloat16": 2e-2}
 # two cuts of the same request through the same engine (in bfloat16 a step of few rows takes other product kernels
 # than a step of many, whose results are rounded to bfloat16 where the others' stay float partial sums)
-CUT_TOLERANCE = {"float32": 3e-6, "bfloat16": 1.5e-1}
+# (in 32-bit too a cut changes the order of sums: a sequence that brings many tokens takes the memory's sliced walk)
+CUT_TOLERANCE = {"float32": 1e-5, "bfloat16": 1.5e-1}
 
 
 def make_model(folder, raw_config, seed, std=0.08, norm_std=0.1):

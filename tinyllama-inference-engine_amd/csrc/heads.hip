@@ -34,23 +34,41 @@ head_combine_kernel(const float* __restrict__ a, int heads, int dv, int pair_gro
     const float second = row[((static_cast<size_t>(2 * g + 1) * parts + p) * pair_group + i) * piece + inside];
     return first - lambda * second;
   };
-  float squares = 0.f;
-  for (int e = lane; e < dv; e += 64) {
-    const float o = value(e);
-    squares += o * o;
-  }
-  const float r = 1.f / sqrtf(wave_sum(squares) / static_cast<float>(dv) + eps);
-  for (int e = lane; e < dv; e += 64) {
-    const float o = value(e);
+  auto emit = [&](int e, float normed) {
     const int c = h * dv + e;
-    float v = o * r * mult;
+    float v = normed * mult;
     if (weight != nullptr) v *= to_float(weight[c]);
     if (gate != nullptr) {
       const float z = sum_splits(gate + static_cast<size_t>(t) * gate_row + gate_col + c, gate_nsplit, gate_split_stride);
       v *= 1.f / (1.f + expf(-z));
     }
     out[static_cast<size_t>(t) * heads * dv + c] = from_float<A>(v);
+  };
+  // a lane's dims (lane, lane + 64, ...) are read once and kept, up to 512 dims a head; beyond, read again
+  constexpr int kKept = 8;
+  const bool fits = dv <= 64 * kKept;
+  float kept[kKept];
+  float squares = 0.f;
+#pragma unroll
+  for (int i = 0; i < kKept; ++i) {
+    const int e = lane + 64 * i;
+    kept[i] = fits && e < dv ? value(e) : 0.f;
+    squares += kept[i] * kept[i];
   }
+  if (!fits) {
+    for (int e = lane; e < dv; e += 64) {
+      const float o = value(e);
+      squares += o * o;
+    }
+  }
+  const float r = 1.f / sqrtf(wave_sum(squares) / static_cast<float>(dv) + eps);
+#pragma unroll
+  for (int i = 0; i < kKept; ++i) {
+    const int e = lane + 64 * i;
+    if (fits && e < dv) emit(e, kept[i] * r);
+  }
+  if (fits) return;
+  for (int e = lane; e < dv; e += 64) emit(e, value(e) * r);
 }
 
 }  // namespace tlie

@@ -91,9 +91,24 @@ few_outputs_kernel(const X* __restrict__ x, const W* __restrict__ w, const W* __
 template <typename D, typename A>
 __global__ void __launch_bounds__(256)
 routed_gate_kernel(const D* __restrict__ gate_up, int nsplit, size_t split_stride, const float* __restrict__ scale,
-                   int experts, int block, A* __restrict__ out, int inter) {
+                   int experts, int block, A* __restrict__ out, int inter, bool wide) {
   const int t = blockIdx.x;
   const D* row = gate_up + static_cast<size_t>(t) * 2 * inter;
+  if (wide) {
+    // four columns a thread: eight values in one load, four out in one store (no partial sums, four columns in one
+    // expert's block, rows that start at multiples of 32 bytes)
+    for (int c = (blockIdx.y * 256 + threadIdx.x) * 4; c < inter; c += gridDim.y * 1024) {
+      const int e = c / block;
+      const float s = e < experts ? scale[static_cast<size_t>(t) * experts + e] : 1.f;
+      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (s != 0.f) load8(row + 2 * c, v);
+      A* to = out + static_cast<size_t>(t) * inter + c;
+      if (s == 0.f) store4(to, 0.f, 0.f, 0.f, 0.f);
+      else store4(to, gated_value(s * v[0], s * v[1], kGateSilu, 1.f, 0.f), gated_value(s * v[2], s * v[3], kGateSilu, 1.f, 0.f),
+                  gated_value(s * v[4], s * v[5], kGateSilu, 1.f, 0.f), gated_value(s * v[6], s * v[7], kGateSilu, 1.f, 0.f));
+    }
+    return;
+  }
   for (int c = blockIdx.y * 256 + threadIdx.x; c < inter; c += gridDim.y * 256) {
     const int e = c / block;
     const float s = e < experts ? scale[static_cast<size_t>(t) * experts + e] : 1.f;
@@ -138,14 +153,16 @@ extern "C" int tlie_routed_gate(const void* gate_up, int in_dtype, int nsplit, l
                                 int experts, int block, void* out, int out_dtype, int tokens, int inter, void* stream) {
   if (tokens <= 0 || inter <= 0 || experts < 0 || block <= 0 || nsplit < 1) return kBadArgument;
   if (static_cast<long long>(experts) * block > inter) return kBadArgument;
-  int across = (inter + 255) / 256;
+  const bool wide = nsplit == 1 && (inter & 3) == 0 && (block & 3) == 0 &&
+                    ((reinterpret_cast<uintptr_t>(gate_up) | reinterpret_cast<uintptr_t>(out)) & 31) == 0;
+  int across = (inter + (wide ? 1023 : 255)) / (wide ? 1024 : 256);
   if (across > 64) across = 64;
   const dim3 grid(tokens, across);
   hipStream_t s = (hipStream_t)stream;
 #define TLIE_CASE(DC, D, AC, A)                                                                                       \
   if (in_dtype == DC && out_dtype == AC) {                                                                            \
     hipLaunchKernelGGL((routed_gate_kernel<D, A>), grid, dim3(256), 0, s, (const D*)gate_up, nsplit,                   \
-                       (size_t)split_stride, scale, experts, block, (A*)out, inter);                                  \
+                       (size_t)split_stride, scale, experts, block, (A*)out, inter, wide);                                  \
     return launch_status();                                                                                           \
   }
   TLIE_CASE(kF32, float, kF32, float)
