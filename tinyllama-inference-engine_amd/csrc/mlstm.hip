@@ -42,12 +42,20 @@ mlstm_gates_kernel(const float* __restrict__ gates, float* __restrict__ values, 
   if (first >= last) return;
   float* m_place = state + (static_cast<size_t>(slot) * heads + h) * head_floats + m_offset;
   float m = *m_place;
+  // (a chunk's two pre-activations are asked for while the chunk before it is worked on)
+  float pre_i = first + lane < last ? gates[static_cast<size_t>(first + lane) * 2 * heads + h] : 0.f;
+  float pre_f = first + lane < last ? gates[static_cast<size_t>(first + lane) * 2 * heads + heads + h] : 0.f;
   for (int t0 = first; t0 < last; t0 += 64) {
     const int t = t0 + lane, count = min(64, last - t0);
+    const float now_i = pre_i, now_f = pre_f;
+    if (t + 64 < last) {
+      pre_i = gates[static_cast<size_t>(t + 64) * 2 * heads + h];
+      pre_f = gates[static_cast<size_t>(t + 64) * 2 * heads + heads + h];
+    }
     float ig = 0.f, fg = 0.f;
     if (lane < count) {
-      ig = cap * tanhf(gates[static_cast<size_t>(t) * 2 * heads + h] / cap);
-      const float x = cap * tanhf(gates[static_cast<size_t>(t) * 2 * heads + heads + h] / cap);
+      ig = cap * tanhf(now_i / cap);
+      const float x = cap * tanhf(now_f / cap);
       fg = fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
     }
     // m' = max(m + f, i) token by token is a chain of the maps m -> max(m + F, I); two in a row are one of the same
@@ -243,10 +251,22 @@ mlstm_carry_kernel(float* __restrict__ parts, float* __restrict__ state, const i
   float* st = state + (static_cast<size_t>(slot) * heads * tiles + unit) * tile_floats;
   for (int e = blockIdx.z * 256 + threadIdx.x; e < elements; e += gridDim.z * 256) {
     float value = st[e];
-    for (int c = 0; c < used; ++c) {
-      float* part = parts + ((static_cast<size_t>(seq) * slices + c) * heads * tiles + unit) * tile_floats;
-      const float end = part[e], keeps = part[elements];
-      part[e] = value;
+    const size_t stride = static_cast<size_t>(heads) * tiles * tile_floats;
+    float* part = parts + (static_cast<size_t>(seq) * slices * heads * tiles + unit) * tile_floats;
+    int c = 0;
+    for (; c + 4 <= used; c += 4) {                    // (four slices' ends asked for together; the chain is the sums' only)
+      float end[4], keeps[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) end[u] = part[(c + u) * stride + e], keeps[u] = part[(c + u) * stride + elements];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        part[(c + u) * stride + e] = value;
+        value = keeps[u] * value + end[u];
+      }
+    }
+    for (; c < used; ++c) {
+      const float end = part[c * stride + e], keeps = part[c * stride + elements];
+      part[c * stride + e] = value;
       value = keeps * value + end;
     }
     if (used > 0) st[e] = value;

@@ -18,7 +18,21 @@ template <typename D, typename A>
 __global__ void __launch_bounds__(256)
 residual_update_kernel(float* __restrict__ residual, const D* __restrict__ a, int a_nsplit, size_t a_stride,
                        const D* __restrict__ b, int b_nsplit, size_t b_stride, float mult, size_t count,
-                       A* __restrict__ copy) {
+                       A* __restrict__ copy, bool wide) {
+  if (wide) {
+    // eight elements a thread and load (no partial sums, a count that is a multiple of 8, addresses at multiples of 32 bytes)
+    for (size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 8; i < count; i += static_cast<size_t>(gridDim.x) * 2048) {
+      float x[8], av[8], bv[8];
+      load8(residual + i, x);
+      load8(a + i, av);
+      if (b != nullptr) load8(b + i, bv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] += mult * (b != nullptr ? av[j] + bv[j] : av[j]);
+      store8(residual + i, x);
+      if (copy != nullptr) store8(copy + i, x);
+    }
+    return;
+  }
   for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += static_cast<size_t>(gridDim.x) * 256) {
     float delta = sum_splits(a + i, a_nsplit, a_stride);
     if (b != nullptr) delta += sum_splits(b + i, b_nsplit, b_stride);
@@ -64,14 +78,17 @@ extern "C" int tlie_residual_update(float* residual, const void* a, int a_nsplit
                                     int b_nsplit, long long b_stride, int in_dtype, float mult, long long count, void* copy,
                                     int copy_dtype, void* stream) {
   if (count <= 0 || a == nullptr || a_nsplit < 1 || (b != nullptr && b_nsplit < 1)) return kBadArgument;
-  long long blocks = (count + 255) / 256;
+  const bool wide = a_nsplit == 1 && (b == nullptr || b_nsplit == 1) && (count & 7) == 0 &&
+                    ((reinterpret_cast<uintptr_t>(residual) | reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+                      reinterpret_cast<uintptr_t>(copy)) & 31) == 0;
+  long long blocks = wide ? (count / 8 + 255) / 256 : (count + 255) / 256;
   if (blocks > 65535LL * 16) blocks = 65535LL * 16;
   hipStream_t s = (hipStream_t)stream;
 #define TLIE_CASE(DC, D, AC, A)                                                                                       \
   if (in_dtype == DC && copy_dtype == AC) {                                                                           \
     hipLaunchKernelGGL((residual_update_kernel<D, A>), dim3((unsigned)blocks), dim3(256), 0, s, residual, (const D*)a,  \
                        a_nsplit, (size_t)a_stride, (const D*)b, b_nsplit, (size_t)b_stride, mult, (size_t)count,       \
-                       (A*)copy);                                                                                     \
+                       (A*)copy, wide);                                                                                     \
     return launch_status();                                                                                           \
   }
   TLIE_CASE(kF32, float, kF32, float)
