@@ -591,3 +591,33 @@ def test_the_command_line_and_the_replay_program_run_the_design(setups, tmp_path
         assert_rows(read(0), want[[0, 29]], TOLERANCE[dtype], f"{dtype} step 0")
         assert_rows(read(1), torch.stack([want[30], want_other[20]]), TOLERANCE[dtype], f"{dtype} step 1")
         assert_rows(read(3), torch.stack([want[39], want_other[20]]), TOLERANCE[dtype], f"{dtype} step 3")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["memory_only", "attention_only"])
+def test_models_of_one_kind_of_layer_and_odd_sizes(tmp_path, which, dtype):
+    """A model without any attention layer (no page group at all) at a width that is no multiple of 8, and one without
+    any memory layer (no state area) whose loop runs once and ends with the model's last layer."""
+    if which == "memory_only":
+        raw = {"architecture": "Raketar", "vocab": 77, "width": 100, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+               "token_side": {"dim": 5}, "loop": {"start": 0, "stop": 2, "times": 2},
+               "layers": [{"type": "mlstm", "mixer": {"heads": 2, "dim": 20, "vdim": 30, "gate_cap": 8.0}, "mlp": {"kind": "dense", "ff": 52}},
+                          {"type": "mlstm", "mixer": {"heads": 5, "dim": 4, "vdim": 7, "gate_cap": 20.0}, "mlp": None}]}
+    else:
+        rot = {"base": 5000.0, "dims": 16, "scaling": {"factor": 3.0}}
+        raw = {"architecture": "Raketar", "vocab": 90, "width": 64, "norm": {"eps": 1e-6}, "residual_mult": 1.5,
+               "loop": {"start": 1, "stop": 2, "times": 1},
+               "layers": [{"type": "attention", "mixer": {"heads": 2, "kv_heads": 2, "dim": 16, "vdim": 16, "scale": 0.25, "diff": 0.0, "rot": rot},
+                           "mlp": {"kind": "moe", "expert": {"ff": 16}, "router": {"experts": 70, "top": 4}, "shared": {"ff": 8}}},
+                          {"type": "attention", "mixer": {"heads": 8, "kv_heads": 2, "dim": 16, "vdim": 64, "scale": 0.25, "diff": 0.9, "rot": rot},
+                           "mlp": None}]}
+    folder = make_model(tmp_path, raw, seed=17)
+    config, weights = load_plain(folder)
+    tokens = tokens_of(19, 140, raw["vocab"])
+    want = plain.forward(config, weights, tokens)[0]
+    from tlie_amd import Engine
+    engine = Engine(folder, dtype=dtype, max_tokens=320, page_size=16, max_requests=2)
+    for cuts in ([140], [100] + [1] * 40, [3, 64, 2, 1]):
+        assert_rows(run_cut(engine, "a", tokens, cuts), want, TOLERANCE[dtype], f"{which} {dtype} cuts {cuts[:4]}")
+    engine.cache.check()
+    assert engine.generate([tokens[:12], tokens[20:25]], max_tokens=4, chunk_size=8) is not None
